@@ -11,10 +11,13 @@ from ..registry import ARCHITECTURES
 from .engine import EngineConfig, parse_dtype
 from .spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
 from .gemma2 import ConfigError, Gemma2Config
+from .zenuzen import ZenuzenConfig
 
 
 def architecture_name(d: Mapping[str, Any]) -> str:
     archs = d.get("architectures")
+    if not archs and isinstance(d.get("architecture"), str):   # (some folders name one architecture, as a string)
+        return d["architecture"]
     if not archs or not isinstance(archs, (list, tuple)):
         raise ConfigError('config.json: key "architectures" is missing or empty; known: '
                           + ", ".join(ARCHITECTURES.keys()))
@@ -35,4 +38,4 @@ def load_config(model_dir: str):
 
 
 __all__ = ["EngineConfig", "parse_dtype", "LayerSpec", "ModelSpec", "PartSpec", "ScheduleEntry",
-           "ConfigError", "Gemma2Config", "architecture_name", "config_from_dict", "load_config"]
+           "ConfigError", "Gemma2Config", "ZenuzenConfig", "architecture_name", "config_from_dict", "load_config"]

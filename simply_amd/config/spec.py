@@ -27,11 +27,12 @@ class PartSpec:
 
 @dataclasses.dataclass(frozen=True)
 class LayerSpec:
-    """A block: an arrangement (`block.kind`) of a mixer, a feed-forward and norms."""
+    """A block: an arrangement (`block.kind`) of a mixer, a feed-forward (None: the layer has none, for block
+    arrangements that allow it) and norms."""
 
     block: PartSpec
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: "PartSpec | None"
     norms: Mapping[str, PartSpec] = dataclasses.field(default_factory=dict)
 
 

@@ -265,5 +265,62 @@ int gemm_tiled(const void* A, int64_t lda, const void* W, void* C, int c_dtype, 
 int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
                             const int* block_table, int table_stride, const int* token_seq, const int* positions,
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,
-                            float soft_cap, hipStream_t stream);
+                            float soft_cap, hipStream_t stream, int hd_v = 0, float scale = 1.f,
+                            const void* sinks = nullptr, int sinks_dtype = 0);
 }  // namespace sa
+
+extern "C" {
+// Attention as sa_paged_attention, for mixers whose values have another size than their keys, whose scores are
+// multiplied by `scale` (before the cap, if there is one) and whose softmax may hold one more term per query head,
+// exp(sinks[h]), that has no key and no value (sinks null: none).  Value pages are [num_pages, Kh, hd_v, page_size];
+// out rows hold H * hd_v elements.
+int sa_paged_attention_sink(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
+                            const int* block_table, int table_stride, const int* token_seq, const int* positions,
+                            void* out, int64_t out_stride, int T, int H, int Kh, int hd, int hd_v, int page_size,
+                            int window, float soft_cap, float scale, const void* sinks, int sinks_dtype,
+                            hipStream_t stream);
+
+// residual += mult * norm(y; w) (w null: + mult * y; y null: nothing is added), then, if out is not null, out = the
+// residual in out's type: the sum of a block that norms what a part returns, and the hand-over to a next part that
+// has no norm in front of it.  The norm is y / sqrt(mean(y^2) + eps) * (w + plus_one).
+int sa_residual_add_norm(const void* y, int y_dtype, int64_t y_stride, const void* w, int w_dtype, float eps,
+                         int plus_one, float mult, float* residual, void* out, int out_dtype, int T, int D,
+                         hipStream_t stream);
+
+// out[t, h, :] = (w null ? x[t, h, :] : x[t, h, :] / sqrt(mean(x[t, h, :]^2) + eps) * w) * gate(g[t, h, :]) for H
+// heads of `size` elements; w [size] is shared by the heads; gate 0: sigmoid, 1: silu.  out may be x.
+int sa_gated_heads(const void* x, int x_dtype, int64_t x_stride, const void* g, int g_dtype, int64_t g_stride,
+                   const void* w, int w_dtype, float eps, int gate, void* out, int out_dtype, int64_t out_stride, int T,
+                   int H, int size, hipStream_t stream);
+
+// x[t, n] = act(x[t, n]) in place (activation codes of activations.h).
+int sa_activation(void* x, int dtype, int64_t stride, int T, int N, int act, hipStream_t stream);
+
+// Rows [H * dk queries | K * dk keys | K * dv values | ...] of a fused projection: queries and keys are rotated on
+// their first rot_dims dimensions (pairs (i, i + rot_dims / 2), angle position * inv_freq[i]) and then divided by
+// sqrt(mean(x^2) + eps) over the head (eps < 0: not); queries go back in place, keys into the key pages; values
+// become (1 - *lambda) v + *lambda v_first[t] (v_first null: stay) and go into the value pages
+// [num_pages, K, dv, page_size].  k_pages null: nothing is written.
+int sa_qk_norm_rope_cache_write(void* proj, int dtype, int64_t row_stride, const int* positions, const float* inv_freq,
+                                int rot_dims, float eps, const void* v_first, int64_t v_first_stride,
+                                const void* lambda, int lambda_dtype, const int64_t* slot_mapping, void* k_pages,
+                                void* v_pages, int T, int H, int K, int dk, int dv, int page_size, hipStream_t stream);
+
+// y[t, c] = silu(sum_j taps[c, j] x[t - (n - 1 - j), c]) over each request's tokens (seq_meta [S, 4]: state slot,
+// first row, rows, first position), with the inputs before the step's first row taken from tails[slot]
+// [n - 1][C] float32, oldest first.  update_tails: afterwards the tails hold each request's last n - 1 inputs.
+int sa_short_conv_silu(const void* x, int x_dtype, int64_t x_stride, const void* taps, int taps_dtype, int num_taps,
+                       float* tails, int64_t tail_stride, const int* seq_meta, int num_seqs, int max_q_len, float* y,
+                       int C, int update_tails, hipStream_t stream);
+
+// In place on qkv [T, C] float32 = [G q heads | G k heads | values]: q and k heads to unit length
+// (x / sqrt(sum(x^2) + 1e-6)), q also times dk^(-1/2).  gates [T, 2 H] receives beta = sigmoid(b) and
+// g = exp(-exp(a_log) * softplus(a + dt_bias)) from ab [T, a (H) | b (H)].
+int sa_delta_prepare(float* qkv, int T, int C, int G, int dk, const void* ab, int ab_dtype, int64_t ab_stride,
+                     const void* a_log, const void* dt_bias, int vec_dtype, int H, float* gates, hipStream_t stream);
+
+// The gated delta rule over each request's tokens, from and into state[slot] [H][dk][dv] float32: per head
+// S <- g S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.  Value head h reads q/k head h / (H / G).
+int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, const float* gates, int H, float* state,
+                  int64_t state_stride, const int* seq_meta, int num_seqs, float* out, hipStream_t stream);
+}

@@ -26,8 +26,8 @@ template <typename T>
 __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_seq,
-    const int* __restrict__ positions, T* __restrict__ out, int64_t out_stride, int Kh, int G, int hd, int page_size,
-    int window, float soft_cap) {
+    const int* __restrict__ positions, T* __restrict__ out, int64_t out_stride, int Kh, int G, int hd, int hd_v,
+    int page_size, int window, float soft_cap, float scale, const void* __restrict__ sinks, int sinks_dtype) {
   extern __shared__ float smem[];
   float* q_s = smem;                      // [G][hd]
   float* s_s = q_s + G * hd;              // [G][kChunk] scores, then probabilities
@@ -95,6 +95,7 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
             s += __shfl_xor(s, 1, kWave);
             s += __shfl_xor(s, 2, kWave);
             if (part == 0) {
+              s *= scale;
               if (soft_cap > 0.f) s = soft_cap * tanhf(s / soft_cap);
               s_s[(g0 + g) * kChunk + j] = valid ? s : -INFINITY;
             }
@@ -125,14 +126,14 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
 #pragma unroll
       for (int s = 0; s < kMaxDimsPerThread; ++s) {
         const int d = tid + s * kThreads;
-        if (d < hd) {
+        if (d < hd_v) {
 #pragma unroll
           for (int g = 0; g < 8; ++g)
             if (g < gn) acc[s][g] *= a_s[g0 + g];
           for (int j = jlo; j < jhi; ++j) {
             const int key = c0 + j;
             const float v = to_float(
-                v_pages[((static_cast<size_t>(page_s[j]) * Kh + kh) * hd + d) * page_size + key % page_size]);
+                v_pages[((static_cast<size_t>(page_s[j]) * Kh + kh) * hd_v + d) * page_size + key % page_size]);
 #pragma unroll
             for (int g = 0; g < 8; ++g)
               if (g < gn) acc[s][g] = fmaf(s_s[(g0 + g) * kChunk + j], v, acc[s][g]);
@@ -144,12 +145,16 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
 #pragma unroll
     for (int s = 0; s < kMaxDimsPerThread; ++s) {
       const int d = tid + s * kThreads;
-      if (d < hd) {
+      if (d < hd_v) {
 #pragma unroll
         for (int g = 0; g < 8; ++g)
-          if (g < gn)
-            out[static_cast<size_t>(t) * out_stride + static_cast<size_t>(kh * G + g0 + g) * hd + d] =
-                from_float<T>(acc[s][g] / l_s[g0 + g]);
+          if (g < gn) {
+            // a sink is one more term of the softmax's sum, exp(sink - maximum), without a value
+            float l = l_s[g0 + g];
+            if (sinks != nullptr) l += expf(load_f(sinks, sinks_dtype, kh * G + g0 + g) - m_s[g0 + g]);
+            out[static_cast<size_t>(t) * out_stride + static_cast<size_t>(kh * G + g0 + g) * hd_v + d] =
+                from_float<T>(acc[s][g] / l);
+          }
       }
     }
   }
@@ -158,10 +163,12 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
 int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
                             const int* block_table, int table_stride, const int* token_seq, const int* positions,
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,
-                            float soft_cap, hipStream_t stream) {
+                            float soft_cap, hipStream_t stream, int hd_v, float scale, const void* sinks,
+                            int sinks_dtype) {
   const int G = H / Kh;
-  if (hd > kThreads * kMaxDimsPerThread) {
-    set_error("paged_attention: head size %d is above the largest supported (%d)", hd, kThreads * kMaxDimsPerThread);
+  if (hd_v <= 0) hd_v = hd;
+  if (hd_v > kThreads * kMaxDimsPerThread) {
+    set_error("paged_attention: value size %d is above the largest supported (%d)", hd_v, kThreads * kMaxDimsPerThread);
     return 1;
   }
   const size_t smem = sizeof(float) * (static_cast<size_t>(G) * hd + static_cast<size_t>(G) * kChunk + 3 * G) +
@@ -176,12 +183,12 @@ int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const vo
     paged_attention_generic_kernel<float><<<grid, kThreads, smem, stream>>>(
         static_cast<const float*>(q), q_stride, static_cast<const float*>(k_pages),
         static_cast<const float*>(v_pages), block_table, table_stride, token_seq, positions, static_cast<float*>(out),
-        out_stride, Kh, G, hd, page_size, window, soft_cap);
+        out_stride, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype);
   else
     paged_attention_generic_kernel<bf16><<<grid, kThreads, smem, stream>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages),
-        block_table, table_stride, token_seq, positions, static_cast<bf16*>(out), out_stride, Kh, G, hd, page_size,
-        window, soft_cap);
+        block_table, table_stride, token_seq, positions, static_cast<bf16*>(out), out_stride, Kh, G, hd, hd_v, page_size,
+        window, soft_cap, scale, sinks, sinks_dtype);
   return check_launch("paged_attention_generic");
 }
 

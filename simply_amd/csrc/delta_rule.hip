@@ -1,0 +1,239 @@
+// A recurrent mixer with a matrix state per head (the gated delta rule) over a ragged batch of requests:
+//
+//   short causal convolution per channel, then silu          short_conv_silu_kernel (+ conv_tail_update_kernel)
+//   q, k to unit length, q / sqrt(size); beta and decay      delta_prepare_kernel
+//   S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q   delta_rule_kernel
+//
+// A request's tokens of this step are rows first .. first + count - 1 of the step (seq_meta [S, 4]: state slot,
+// first row, count, position of the first); what earlier steps left is the slot's state: the matrix S per head and
+// the last taps - 1 inputs of the convolution.  Everything is 32-bit; sums run in a fixed order that depends on
+// nothing but the sizes, so a token's result is the same however the tokens are cut into steps and whatever else
+// is in the batch.
+#include "api.h"
+#include "common.h"
+
+namespace sa {
+
+constexpr int kMaxTaps = 8;
+constexpr int kConvTokens = 16;  // tokens that one thread of the convolution walks through
+
+// y[t, c] = silu(sum_j taps[c, j] * x[t - (n - 1 - j), c]) with x before the step's first token taken from the
+// request's tail [n - 1][C] (oldest first).  A thread takes one channel and kConvTokens consecutive tokens.
+__global__ __launch_bounds__(kWave) void short_conv_silu_kernel(
+    const void* __restrict__ x, int x_dtype, int64_t x_stride, const void* __restrict__ taps, int taps_dtype, int n,
+    const float* __restrict__ tails, int64_t tail_stride, const int* __restrict__ seq_meta, float* __restrict__ y,
+    int C) {
+  const int* meta = seq_meta + 4 * blockIdx.y;
+  const int slot = meta[0], first = meta[1], count = meta[2];
+  const int j0 = blockIdx.x * kConvTokens;
+  const int c = blockIdx.z * kWave + threadIdx.x;
+  if (j0 >= count || c >= C) return;
+  float w[kMaxTaps], win[kMaxTaps];   // win[i]: input at token j - (n - 1 - i)
+#pragma unroll
+  for (int i = 0; i < kMaxTaps; ++i) w[i] = i < n ? load_f(taps, taps_dtype, static_cast<size_t>(c) * n + i) : 0.f;
+  const float* tail = tails + static_cast<size_t>(slot) * tail_stride;
+  auto input = [&](int j) -> float {   // j: token of the request in this step; negative: before the step
+    if (j >= 0) return load_f(x, x_dtype, static_cast<size_t>(first + j) * x_stride + c);
+    return tail[static_cast<size_t>(n - 1 + j) * C + c];
+  };
+#pragma unroll
+  for (int i = 0; i < kMaxTaps; ++i) win[i] = (i >= 1 && i < n) ? input(j0 - (n - i)) : 0.f;   // win[1..n-1]: the n - 1 before j0
+  const int jn = count - j0 < kConvTokens ? count - j0 : kConvTokens;
+  for (int j = 0; j < jn; ++j) {
+#pragma unroll
+    for (int i = 0; i + 1 < kMaxTaps; ++i) win[i] = win[i + 1];
+    // (the newest sits at win[n - 1]: entries from n on are never read)
+    const float cur = input(j0 + j);
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i)
+      if (i == n - 1) win[i] = cur;
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i)
+      if (i < n) acc = fmaf(w[i], win[i], acc);
+    y[static_cast<size_t>(first + j0 + j) * C + c] = acc / (1.f + expf(-acc));
+  }
+}
+
+// The tails after the step: the last n - 1 inputs of every request, from this step's rows and, where the step brought
+// fewer than n - 1 tokens, from the old tail.  A thread takes one channel of one request; it reads old entries only
+// at places that it has not written yet.
+__global__ __launch_bounds__(kWave) void conv_tail_update_kernel(const void* __restrict__ x, int x_dtype,
+                                                                 int64_t x_stride, int n, float* __restrict__ tails,
+                                                                 int64_t tail_stride, const int* __restrict__ seq_meta,
+                                                                 int C) {
+  const int* meta = seq_meta + 4 * blockIdx.y;
+  const int slot = meta[0], first = meta[1], count = meta[2];
+  const int c = blockIdx.x * kWave + threadIdx.x;
+  if (c >= C || count <= 0) return;
+  float* tail = tails + static_cast<size_t>(slot) * tail_stride;
+  for (int i = 0; i < n - 1; ++i) {
+    const int j = count - (n - 1) + i;   // token of this step that becomes entry i; negative: an old entry
+    tail[static_cast<size_t>(i) * C + c] = j >= 0 ? load_f(x, x_dtype, static_cast<size_t>(first + j) * x_stride + c)
+                                                  : tail[static_cast<size_t>(n - 1 + j) * C + c];
+  }
+}
+
+// Per (token, unit): units 0 .. 2 G - 1 are the q and k heads of qkv [T, C] (q heads first), each made a unit vector
+// x / sqrt(sum(x^2) + 1e-6), the queries also times size^(-1/2); unit 2 G computes, for every value head h,
+// beta = sigmoid(b) and g = exp(-exp(A_log) * softplus(a + dt_bias)) into gates [T, 2 H] (beta first).
+__global__ __launch_bounds__(kWave) void delta_prepare_kernel(float* __restrict__ qkv, int C, int G, int dk,
+                                                              const void* __restrict__ ab, int ab_dtype,
+                                                              int64_t ab_stride, const void* __restrict__ a_log,
+                                                              const void* __restrict__ dt_bias, int vec_dtype, int H,
+                                                              float* __restrict__ gates) {
+  const int t = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
+  if (unit < 2 * G) {
+    float* head = qkv + static_cast<size_t>(t) * C + static_cast<size_t>(unit) * dk;
+    float ss = 0.f;
+    for (int i = lane; i < dk; i += kWave) ss = fmaf(head[i], head[i], ss);
+    ss = wave_sum(ss);
+    float r = 1.f / sqrtf(ss + 1e-6f);
+    if (unit < G) r *= 1.f / sqrtf(static_cast<float>(dk));
+    for (int i = lane; i < dk; i += kWave) head[i] *= r;
+    return;
+  }
+  for (int h = lane; h < H; h += kWave) {
+    const float a = load_f(ab, ab_dtype, static_cast<size_t>(t) * ab_stride + h);
+    const float b = load_f(ab, ab_dtype, static_cast<size_t>(t) * ab_stride + H + h);
+    const float z = a + load_f(dt_bias, vec_dtype, h);
+    const float sp = z > 30.f ? z : log1pf(expf(z));
+    gates[static_cast<size_t>(t) * 2 * H + h] = 1.f / (1.f + expf(-b));
+    gates[static_cast<size_t>(t) * 2 * H + H + h] = expf(-expf(load_f(a_log, vec_dtype, h)) * sp);
+  }
+}
+
+// The recurrence.  A workgroup of 256 threads takes 64 columns of one head's state for one request: four lanes
+// share a column, lane `part` of them holding rows part, part + 4, ... of it in registers (DK / 4 of them).  The
+// step's q and k of kRuleTokens tokens at a time go through LDS.  Columns are independent of each other, rows are
+// summed within a lane in increasing order and then across the four lanes in a fixed order.
+constexpr int kRuleTokens = 16;
+__device__ __forceinline__ float quad_sum(float v) {
+  v += lane_exchange<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+  v += lane_exchange<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  return v;
+}
+
+template <int DK>
+__global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ qkv, int C, int G, int dk, int dv,
+                                                         const float* __restrict__ gates, int H,
+                                                         float* __restrict__ state, int64_t state_stride,
+                                                         const int* __restrict__ seq_meta, float* __restrict__ out) {
+  constexpr int R = DK / 4;
+  __shared__ float qs[kRuleTokens][DK], ks[kRuleTokens][DK], vs[kRuleTokens][64], bg[kRuleTokens][2];
+  const int* meta = seq_meta + 4 * blockIdx.x;
+  const int slot = meta[0], first = meta[1], count = meta[2];
+  const int h = blockIdx.y, tid = threadIdx.x;
+  const int col = blockIdx.z * 64 + tid / 4, part = tid % 4;
+  const bool live = col < dv;
+  const int qk_head = h / (H / G);
+  float* S = state + static_cast<size_t>(slot) * state_stride + static_cast<size_t>(h) * dk * dv;   // [dk][dv]
+  float s[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int i = r * 4 + part;
+    s[r] = (live && i < dk) ? S[static_cast<size_t>(i) * dv + col] : 0.f;
+  }
+  const int v_at = 2 * G * dk + h * dv;
+  for (int t0 = 0; t0 < count; t0 += kRuleTokens) {
+    const int tn = count - t0 < kRuleTokens ? count - t0 : kRuleTokens;
+    __syncthreads();
+    for (int idx = tid; idx < tn * DK; idx += 256) {
+      const int j = idx / DK, i = idx % DK;
+      const float* row = qkv + static_cast<size_t>(first + t0 + j) * C;
+      qs[j][i] = i < dk ? row[qk_head * dk + i] : 0.f;
+      ks[j][i] = i < dk ? row[(G + qk_head) * dk + i] : 0.f;
+    }
+    for (int idx = tid; idx < tn * 64; idx += 256) {
+      const int j = idx / 64, c = blockIdx.z * 64 + idx % 64;
+      vs[j][idx % 64] = c < dv ? qkv[static_cast<size_t>(first + t0 + j) * C + v_at + c] : 0.f;
+    }
+    if (tid < 2 * tn) bg[tid / 2][tid % 2] = gates[static_cast<size_t>(first + t0 + tid / 2) * 2 * H + (tid % 2) * H + h];
+    __syncthreads();
+    for (int j = 0; j < tn; ++j) {
+      const size_t t = static_cast<size_t>(first + t0 + j);
+      const float beta = bg[j][0], g = bg[j][1];
+      const float v = vs[j][tid / 4];
+      float dot = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        s[r] *= g;
+        dot = fmaf(s[r], ks[j][r * 4 + part], dot);
+      }
+      dot = quad_sum(dot);
+      const float u = beta * (v - dot);
+      float o = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        s[r] = fmaf(ks[j][r * 4 + part], u, s[r]);
+        o = fmaf(s[r], qs[j][r * 4 + part], o);
+      }
+      o = quad_sum(o);
+      if (live && part == 0) out[t * (static_cast<size_t>(H) * dv) + static_cast<size_t>(h) * dv + col] = o;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int i = r * 4 + part;
+    if (live && i < dk) S[static_cast<size_t>(i) * dv + col] = s[r];
+  }
+}
+
+}  // namespace sa
+
+using namespace sa;
+
+extern "C" int sa_short_conv_silu(const void* x, int x_dtype, int64_t x_stride, const void* taps, int taps_dtype,
+                                  int num_taps, float* tails, int64_t tail_stride, const int* seq_meta, int num_seqs,
+                                  int max_q_len, float* y, int C, int update_tails, hipStream_t stream) {
+  if (num_seqs == 0 || max_q_len == 0) return 0;
+  SA_REQUIRE(num_seqs > 0 && max_q_len > 0 && C > 0 && x != nullptr && taps != nullptr && tails != nullptr &&
+                 seq_meta != nullptr && y != nullptr,
+             "short_conv_silu: bad sizes S=%d q=%d C=%d", num_seqs, max_q_len, C);
+  SA_REQUIRE(num_taps >= 1 && num_taps <= kMaxTaps, "short_conv_silu: 1 to %d taps, got %d", kMaxTaps, num_taps);
+  SA_REQUIRE(x_stride >= C && tail_stride >= static_cast<int64_t>(num_taps - 1) * C,
+             "short_conv_silu: a stride is below what the %d channels need", C);
+  SA_REQUIRE(num_seqs <= 65535 && (C + kWave - 1) / kWave <= 65535, "short_conv_silu: too many requests or channels");
+  const dim3 grid((max_q_len + kConvTokens - 1) / kConvTokens, num_seqs, (C + kWave - 1) / kWave);
+  short_conv_silu_kernel<<<grid, kWave, 0, stream>>>(x, x_dtype, x_stride, taps, taps_dtype, num_taps, tails,
+                                                     tail_stride, seq_meta, y, C);
+  if (update_tails && num_taps > 1)
+    conv_tail_update_kernel<<<dim3((C + kWave - 1) / kWave, num_seqs), kWave, 0, stream>>>(
+        x, x_dtype, x_stride, num_taps, tails, tail_stride, seq_meta, C);
+  return check_launch("short_conv_silu");
+}
+
+extern "C" int sa_delta_prepare(float* qkv, int T, int C, int G, int dk, const void* ab, int ab_dtype, int64_t ab_stride,
+                                const void* a_log, const void* dt_bias, int vec_dtype, int H, float* gates,
+                                hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(T > 0 && G > 0 && dk > 0 && H > 0 && C >= 2 * G * dk && H % G == 0 && ab_stride >= 2 * H,
+             "delta_prepare: bad sizes T=%d C=%d G=%d dk=%d H=%d", T, C, G, dk, H);
+  SA_REQUIRE(qkv != nullptr && ab != nullptr && a_log != nullptr && dt_bias != nullptr && gates != nullptr,
+             "delta_prepare: a null pointer");
+  SA_REQUIRE(2 * G + 1 <= 65535, "delta_prepare: too many heads");
+  delta_prepare_kernel<<<dim3(T, 2 * G + 1), kWave, 0, stream>>>(qkv, C, G, dk, ab, ab_dtype, ab_stride, a_log, dt_bias,
+                                                                 vec_dtype, H, gates);
+  return check_launch("delta_prepare");
+}
+
+extern "C" int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, const float* gates, int H, float* state,
+                             int64_t state_stride, const int* seq_meta, int num_seqs, float* out, hipStream_t stream) {
+  if (num_seqs == 0) return 0;
+  SA_REQUIRE(num_seqs > 0 && G > 0 && H > 0 && H % G == 0 && dk > 0 && dv > 0 && C >= 2 * G * dk + H * dv,
+             "delta_rule: bad sizes S=%d C=%d G=%d H=%d dk=%d dv=%d", num_seqs, C, G, H, dk, dv);
+  SA_REQUIRE(dk <= 256, "delta_rule: key size %d is above 256", dk);
+  SA_REQUIRE(state_stride >= static_cast<int64_t>(H) * dk * dv, "delta_rule: the state rows are too short");
+  SA_REQUIRE(qkv != nullptr && gates != nullptr && state != nullptr && seq_meta != nullptr && out != nullptr,
+             "delta_rule: a null pointer");
+  SA_REQUIRE(H <= 65535 && (dv + 63) / 64 <= 65535, "delta_rule: too many heads or columns");
+  const dim3 grid(num_seqs, H, (dv + 63) / 64);
+#define SA_DELTA_RULE(DK) \
+  delta_rule_kernel<DK><<<grid, 256, 0, stream>>>(qkv, C, G, dk, dv, gates, H, state, state_stride, seq_meta, out)
+  if (dk <= 32) SA_DELTA_RULE(32);
+  else if (dk <= 64) SA_DELTA_RULE(64);
+  else if (dk <= 128) SA_DELTA_RULE(128);
+  else SA_DELTA_RULE(256);
+#undef SA_DELTA_RULE
+  return check_launch("delta_rule");
+}

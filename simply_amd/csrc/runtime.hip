@@ -158,6 +158,25 @@ extern "C" int sa_paged_attention(const void* q, int dtype, int64_t q_stride, co
                                  out, out_stride, T, H, Kh, hd, page_size, window, soft_cap, stream);
 }
 
+extern "C" int sa_paged_attention_sink(const void* q, int dtype, int64_t q_stride, const void* k_pages,
+                                       const void* v_pages, const int* block_table, int table_stride,
+                                       const int* token_seq, const int* positions, void* out, int64_t out_stride, int T,
+                                       int H, int Kh, int hd, int hd_v, int page_size, int window, float soft_cap,
+                                       float scale, const void* sinks, int sinks_dtype, hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(dtype == kF32 || dtype == kBF16, "paged_attention_sink: unknown dtype %d", dtype);
+  SA_REQUIRE(T > 0 && H > 0 && Kh > 0 && hd > 0 && hd_v > 0 && page_size > 0,
+             "paged_attention_sink: bad sizes T=%d H=%d K=%d hd=%d hd_v=%d P=%d", T, H, Kh, hd, hd_v, page_size);
+  SA_REQUIRE(H % Kh == 0, "paged_attention_sink: %d query heads do not split over %d key heads", H, Kh);
+  SA_REQUIRE(q_stride >= static_cast<int64_t>(H) * hd && out_stride >= static_cast<int64_t>(H) * hd_v,
+             "paged_attention_sink: row strides are below heads * head size");
+  SA_REQUIRE(window >= 0 && table_stride > 0, "paged_attention_sink: bad window or table stride");
+  SA_REQUIRE(sinks == nullptr || sinks_dtype == kF32 || sinks_dtype == kBF16, "paged_attention_sink: unknown sink dtype");
+  return paged_attention_generic(q, dtype, q_stride, k_pages, v_pages, block_table, table_stride, token_seq, positions,
+                                 out, out_stride, T, H, Kh, hd, page_size, window, soft_cap, stream, hd_v, scale, sinks,
+                                 sinks_dtype);
+}
+
 extern "C" int sa_paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                                          const int* block_table, int table_stride, const int* seq_meta, int seq_begin,
                                          int seq_count, void* out, int64_t out_stride, int H, int Kh, int hd,

@@ -36,6 +36,9 @@ class StepContext:
     q_lens: list[int]             # tokens of the request in this step
     cu_q_lens: list[int]          # [S + 1] offsets of the requests in the flat batch
     _units: dict = dataclasses.field(default_factory=dict)
+    #: what a layer leaves for later layers of the same step, by a name that the two agree on (the values of the
+    #: step's tokens that a later attention layer mixes into its own): tensors over the step's tokens, gone with the step
+    carry: dict = dataclasses.field(default_factory=dict)
     #: set for a step whose launches are recorded and replayed for later steps: the most keys that any step that
     #: replays them may have (kernels size their plans by `max_kv_len`, which is then this bound)
     kv_bound: int = 0

@@ -673,6 +673,233 @@ def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
                             unit_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits)
 
 
+def paged_attention_sink(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                         token_seq: torch.Tensor, positions: torch.Tensor, num_heads: int, *, scale: float = 1.0,
+                         sinks: torch.Tensor | None = None, window: int | None = None, soft_cap: float | None = None,
+                         out: torch.Tensor | None = None) -> torch.Tensor:
+    """Attention whose values may have another size than its keys (key pages [pages, K, P, dk], value pages
+    [pages, K, dv, P]), with scores times `scale` and, if `sinks` [H] is given, one more term exp(sinks[h]) in every
+    softmax sum that has no value.  q: [T, >= H * dk] rows.  Returns [T, H * dv]."""
+    _dev(q, k_pages, v_pages, block_table, token_seq, positions, sinks, out)
+    q_stride = _rows(q, "paged_attention_sink: q")
+    T = q.shape[0]
+    if k_pages.dim() != 4 or v_pages.dim() != 4 or not k_pages.is_contiguous() or not v_pages.is_contiguous() \
+            or k_pages.dtype != q.dtype or v_pages.dtype != q.dtype:
+        raise KernelError(f"paged_attention_sink: pages must be contiguous 4-D tensors of {q.dtype}")
+    num_pages, Kh, page_size, dk = k_pages.shape
+    dv = v_pages.shape[2]
+    if tuple(v_pages.shape) != (num_pages, Kh, dv, page_size):
+        raise KernelError(f"paged_attention_sink: key pages {tuple(k_pages.shape)} do not go with value pages "
+                          f"{tuple(v_pages.shape)}")
+    if q.shape[1] < num_heads * dk:
+        raise KernelError("paged_attention_sink: query rows are shorter than heads * key size")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("paged_attention_sink: block_table must be int32 [sequences, blocks]")
+    _i32(token_seq, "paged_attention_sink: token_seq", T)
+    _i32(positions, "paged_attention_sink: positions", T)
+    if sinks is not None and (sinks.numel() != num_heads or not sinks.is_contiguous()):
+        raise KernelError(f"paged_attention_sink: {sinks.numel()} sinks for {num_heads} heads")
+    if out is None:
+        out = torch.empty((T, num_heads * dv), dtype=q.dtype, device=q.device)
+    if tuple(out.shape) != (T, num_heads * dv) or out.dtype != q.dtype:
+        raise KernelError("paged_attention_sink: bad output")
+    out_stride = _rows(out, "paged_attention_sink: out")
+    _lib.call("sa_paged_attention_sink", _ptr(q), _code(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+              block_table.stride(0), _ptr(token_seq), _ptr(positions), _ptr(out), out_stride, T, num_heads, Kh, dk, dv,
+              page_size, int(window or 0), float(soft_cap or 0.0), float(scale), _ptr(sinks),
+              _code(sinks) if sinks is not None else 0, _stream())
+    return out
+
+
+# --------------------------------------------------------------------------- norms behind parts, gates
+
+
+def residual_add_norm(y: "torch.Tensor | PartialSums | None", residual: torch.Tensor, *,
+                      weight: torch.Tensor | None = None, eps: float = 0.0, plus_one: bool = False, mult: float = 1.0,
+                      out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None) -> torch.Tensor | None:
+    """residual += mult * norm(y; weight) (weight None: += mult * y; y None: nothing is added).  With out_dtype (or
+    out) the updated residual is also returned in that type: what a next part without a norm in front reads."""
+    if isinstance(y, PartialSums):
+        y = y.materialize()
+    _dev(y, residual, weight, out)
+    T, D = residual.shape
+    if residual.dtype != torch.float32 or not residual.is_contiguous():
+        raise KernelError("residual_add_norm: the residual stream must be contiguous float32")
+    ys = 0
+    if y is not None:
+        if tuple(y.shape) != (T, D):
+            raise KernelError(f"residual_add_norm: y {tuple(y.shape)} does not match the residual {T, D}")
+        ys = _rows(y, "residual_add_norm: y")
+    if weight is not None and (weight.numel() != D or not weight.is_contiguous()):
+        raise KernelError("residual_add_norm: the norm weight does not match the width")
+    if out is None and out_dtype is not None:
+        out = torch.empty((T, D), dtype=out_dtype, device=residual.device)
+    if out is not None and (tuple(out.shape) != (T, D) or not out.is_contiguous()):
+        raise KernelError("residual_add_norm: bad output")
+    if y is None and out is None:
+        return None
+    _lib.call("sa_residual_add_norm", _ptr(y), _code(y) if y is not None else 0, ys, _ptr(weight),
+              _code(weight) if weight is not None else 0, float(eps), int(plus_one), float(mult), _ptr(residual),
+              _ptr(out), _code(out) if out is not None else 0, T, D, _stream())
+    return out
+
+
+GATE_SIGMOID, GATE_SILU = 0, 1
+
+
+def gated_heads(x: torch.Tensor, gate: torch.Tensor, num_heads: int, size: int, *, kind: int,
+                weight: torch.Tensor | None = None, eps: float = 0.0, out_dtype: torch.dtype | None = None,
+                out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t, h] = (x[t, h] normed over the head's `size` entries and times weight [size], if a weight is given,
+    else x[t, h]) * sigmoid(gate[t, h]) or * silu(gate[t, h]).  x, gate: rows of num_heads * size (views with a
+    row stride are fine)."""
+    _dev(x, gate, weight, out)
+    T = x.shape[0]
+    width = num_heads * size
+    xs, gs = _rows(x, "gated_heads: x"), _rows(gate, "gated_heads: gate")
+    if x.shape[1] != width or tuple(gate.shape) != (T, width):
+        raise KernelError(f"gated_heads: rows of {width} expected, got x {tuple(x.shape)} gate {tuple(gate.shape)}")
+    if weight is not None and (weight.numel() != size or not weight.is_contiguous()):
+        raise KernelError("gated_heads: the norm weight has one entry per element of a head")
+    if kind not in (GATE_SIGMOID, GATE_SILU):
+        raise KernelError(f"gated_heads: unknown gate {kind!r}")
+    if out is None:
+        out = torch.empty((T, width), dtype=out_dtype or x.dtype, device=x.device)
+    if tuple(out.shape) != (T, width):
+        raise KernelError("gated_heads: bad output")
+    os_ = _rows(out, "gated_heads: out")
+    _lib.call("sa_gated_heads", _ptr(x), _code(x), xs, _ptr(gate), _code(gate), gs, _ptr(weight),
+              _code(weight) if weight is not None else 0, float(eps), int(kind), _ptr(out), _code(out), os_, T,
+              num_heads, size, _stream())
+    return out
+
+
+def activation_(x: torch.Tensor, activation: int) -> torch.Tensor:
+    """x = act(x) in place (an activation code of the ACTIVATIONS registry)."""
+    _dev(x)
+    stride = _rows(x, "activation_: x")
+    _lib.call("sa_activation", _ptr(x), _code(x), stride, x.shape[0], x.shape[1], int(activation), _stream())
+    return x
+
+
+def qk_norm_rope_cache_write(proj: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor | None, rot_dims: int,
+                             eps: float | None, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, *,
+                             v_first: torch.Tensor | None = None, v_mix: torch.Tensor | None = None,
+                             slot_mapping: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
+                             v_pages: torch.Tensor | None = None) -> torch.Tensor:
+    """In place on fused projection rows [H * dk | K * dk | K * dv | ...]: queries and keys rotated on their first
+    rot_dims dimensions (angle position * inv_freq[i] for the pair (i, i + rot_dims / 2)), then divided by their root
+    mean square (eps None: not); values mixed, (1 - v_mix) v + v_mix v_first (v_first [T, K * dv] rows of another
+    layer, v_mix a tensor of one element), keys and values written into the pages."""
+    _dev(proj, positions, inv_freq, v_first, v_mix, slot_mapping, k_pages, v_pages)
+    stride = _rows(proj, "qk_norm_rope_cache_write: proj")
+    T = proj.shape[0]
+    H, K, dk, dv = num_heads, num_kv_heads, key_dim, value_dim
+    if proj.shape[1] < (H + K) * dk + K * dv:
+        raise KernelError(f"qk_norm_rope_cache_write: rows of {proj.shape[1]} are shorter than (H + K) dk + K dv")
+    _i32(positions, "qk_norm_rope_cache_write: positions", T)
+    if rot_dims:
+        if inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rot_dims // 2 \
+                or not inv_freq.is_contiguous() or rot_dims % 2 or rot_dims > dk:
+            raise KernelError("qk_norm_rope_cache_write: inv_freq must be float32 [rot_dims / 2], rot_dims even, <= dk")
+    page_size, vfs = 1, 0
+    if k_pages is not None:
+        if v_pages is None or slot_mapping is None:
+            raise KernelError("qk_norm_rope_cache_write: key pages, value pages and slots come together")
+        if k_pages.dim() != 4 or v_pages.dim() != 4 or not k_pages.is_contiguous() or not v_pages.is_contiguous() \
+                or k_pages.dtype != proj.dtype or v_pages.dtype != proj.dtype:
+            raise KernelError(f"qk_norm_rope_cache_write: pages must be contiguous 4-D tensors of {proj.dtype}")
+        n, _, page_size, _ = k_pages.shape
+        if tuple(k_pages.shape) != (n, K, page_size, dk) or tuple(v_pages.shape) != (n, K, dv, page_size):
+            raise KernelError(f"qk_norm_rope_cache_write: pages {tuple(k_pages.shape)}, {tuple(v_pages.shape)} do not "
+                              f"match {K} heads of key size {dk} and value size {dv}")
+        if slot_mapping.dtype != torch.int64 or slot_mapping.numel() < T or not slot_mapping.is_contiguous():
+            raise KernelError("qk_norm_rope_cache_write: slot_mapping must be int64 [T]")
+    if v_first is not None:
+        if v_mix is None or v_mix.numel() != 1 or v_first.dtype != proj.dtype or v_first.shape[0] != T \
+                or v_first.shape[1] != K * dv:
+            raise KernelError("qk_norm_rope_cache_write: mixed values need a factor of one element and rows "
+                              "[T, K * dv] of the projection's type")
+        vfs = _rows(v_first, "qk_norm_rope_cache_write: v_first")
+    _lib.call("sa_qk_norm_rope_cache_write", _ptr(proj), _code(proj), stride, _ptr(positions), _ptr(inv_freq),
+              int(rot_dims), float(eps) if eps is not None else -1.0, _ptr(v_first), vfs, _ptr(v_mix),
+              _code(v_mix) if v_mix is not None else 0, _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), T, H, K, dk,
+              dv, int(page_size), _stream())
+    return proj
+
+
+# --------------------------------------------------------------------------- recurrent mixers
+
+
+def short_conv_silu(x: torch.Tensor, taps: torch.Tensor, tails: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int,
+                    max_q_len: int, *, update_tails: bool = True, out: torch.Tensor | None = None) -> torch.Tensor:
+    """y[t, c] = silu(sum_j taps[c, j] x[t - (n - 1 - j), c]) along each request's tokens (seq_meta rows: state slot,
+    first row, rows, first position); inputs before the step come from tails [slots, (n - 1) * C] float32, which
+    afterwards hold each request's last n - 1 inputs.  x: [T, C] rows (a view is fine).  Returns float32 [T, C]."""
+    _dev(x, taps, tails, seq_meta, out)
+    stride = _rows(x, "short_conv_silu: x")
+    T, C = x.shape
+    if taps.dim() != 2 or taps.shape[0] != C or not taps.is_contiguous():
+        raise KernelError(f"short_conv_silu: taps {tuple(taps.shape)} for {C} channels")
+    n = taps.shape[1]
+    if tails.dtype != torch.float32 or tails.dim() != 2 or tails.stride(1) != 1 or tails.shape[1] < (n - 1) * C:
+        raise KernelError("short_conv_silu: tails must be float32 [slots, >= (taps - 1) * channels]")
+    if seq_meta.dtype != torch.int32 or seq_meta.dim() != 2 or seq_meta.shape[1] != 4 or not seq_meta.is_contiguous() \
+            or seq_meta.shape[0] < num_seqs:
+        raise KernelError("short_conv_silu: seq_meta must be int32 [S, 4]")
+    if out is None:
+        out = torch.empty((T, C), dtype=torch.float32, device=x.device)
+    if out.dtype != torch.float32 or tuple(out.shape) != (T, C) or not out.is_contiguous():
+        raise KernelError("short_conv_silu: the output must be contiguous float32 [T, C]")
+    _lib.call("sa_short_conv_silu", _ptr(x), _code(x), stride, _ptr(taps), _code(taps), n, _ptr(tails), tails.stride(0),
+              _ptr(seq_meta), int(num_seqs), int(max_q_len), _ptr(out), C, int(update_tails), _stream())
+    return out
+
+
+def delta_prepare(qkv: torch.Tensor, ab: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, num_heads: int,
+                  num_qk_heads: int, key_dim: int) -> torch.Tensor:
+    """In place on qkv float32 [T, C] = [G q heads | G k heads | values]: q and k heads to unit length, q also times
+    key_dim ** -0.5.  Returns gates float32 [T, 2 H]: beta = sigmoid(b), then g = exp(-exp(a_log) softplus(a +
+    dt_bias)), from ab [T, 2 H] = [a | b]."""
+    _dev(qkv, ab, a_log, dt_bias)
+    T, C = qkv.shape
+    H, G = num_heads, num_qk_heads
+    if qkv.dtype != torch.float32 or not qkv.is_contiguous():
+        raise KernelError("delta_prepare: qkv must be contiguous float32")
+    abs_ = _rows(ab, "delta_prepare: ab")
+    if ab.shape[0] != T or ab.shape[1] != 2 * H:
+        raise KernelError(f"delta_prepare: ab {tuple(ab.shape)} is not [T, 2 H]")
+    if a_log.numel() != H or dt_bias.numel() != H or a_log.dtype != dt_bias.dtype or not a_log.is_contiguous() \
+            or not dt_bias.is_contiguous():
+        raise KernelError("delta_prepare: a_log and dt_bias have one entry per head, of one type")
+    gates = torch.empty((T, 2 * H), dtype=torch.float32, device=qkv.device)
+    _lib.call("sa_delta_prepare", _ptr(qkv), T, C, G, key_dim, _ptr(ab), _code(ab), abs_, _ptr(a_log), _ptr(dt_bias),
+              _code(a_log), H, _ptr(gates), _stream())
+    return gates
+
+
+def delta_rule(qkv: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int,
+               num_heads: int, num_qk_heads: int, key_dim: int, value_dim: int) -> torch.Tensor:
+    """The gated delta rule along each request's tokens, from and into state [slots, >= H * dk * dv] float32 (per
+    slot [H][dk][dv]).  qkv float32 [T, C] as `delta_prepare` left it, gates [T, 2 H].  Returns float32 [T, H * dv]."""
+    _dev(qkv, gates, state, seq_meta)
+    T, C = qkv.shape
+    H, G, dk, dv = num_heads, num_qk_heads, key_dim, value_dim
+    if qkv.dtype != torch.float32 or not qkv.is_contiguous() or C < 2 * G * dk + H * dv:
+        raise KernelError("delta_rule: qkv must be contiguous float32 [T, >= 2 G dk + H dv]")
+    if gates.dtype != torch.float32 or tuple(gates.shape) != (T, 2 * H) or not gates.is_contiguous():
+        raise KernelError("delta_rule: gates must be contiguous float32 [T, 2 H]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < H * dk * dv:
+        raise KernelError("delta_rule: the state must be float32 [slots, >= H * dk * dv]")
+    if seq_meta.dtype != torch.int32 or seq_meta.dim() != 2 or seq_meta.shape[1] != 4 or not seq_meta.is_contiguous() \
+            or seq_meta.shape[0] < num_seqs:
+        raise KernelError("delta_rule: seq_meta must be int32 [S, 4]")
+    out = torch.empty((T, H * dv), dtype=torch.float32, device=qkv.device)
+    _lib.call("sa_delta_rule", _ptr(qkv), C, G, dk, dv, _ptr(gates), H, _ptr(state), state.stride(0), _ptr(seq_meta),
+              int(num_seqs), _ptr(out), _stream())
+    return out
+
+
 # --------------------------------------------------------------------------- measurements of the machine
 
 

@@ -21,7 +21,7 @@ from ..weights import binding
 
 def _build_layer(spec: LayerSpec) -> Block:
     mixer = MIXERS.build(spec.mixer.kind, **spec.mixer.params)
-    ffn = FEED_FORWARDS.build(spec.feed_forward.kind, **spec.feed_forward.params)
+    ffn = None if spec.feed_forward is None else FEED_FORWARDS.build(spec.feed_forward.kind, **spec.feed_forward.params)
     norms = {name: NORMS.build(ns.kind, **ns.params) for name, ns in spec.norms.items()}
     return BLOCKS.build(spec.block.kind, mixer, ffn, norms, **spec.block.params)
 
@@ -41,7 +41,8 @@ class DecoderModel:
         out: list[tuple[Part, PartSpec]] = [(self.embedding, self.spec.embedding)]
         for block, ls in zip(self.layers, self.spec.layers):
             out.append((block.mixer, ls.mixer))
-            out.append((block.feed_forward, ls.feed_forward))
+            if ls.feed_forward is not None:
+                out.append((block.feed_forward, ls.feed_forward))
             for name, ns in ls.norms.items():
                 out.append((block.norms[name], ns))
         out.append((self.final_norm, self.spec.final_norm))

@@ -96,3 +96,90 @@ class PagedAttention(Mixer):
             ops.paged_attention(qkv, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq, ctx.positions, H,
                                 window=self.window, soft_cap=self.soft_cap, out=o)
         return ops.gemm(o, self.o_proj, defer_sum=defer_sum)
+
+
+@MIXERS.register("sink_attention")
+class SinkAttention(Mixer):
+    """Grouped-query attention over a paged cache whose values have a size of their own, with the options
+
+      position_encoding  'partial_rope' (or None): only the first dimensions of a head are rotated;
+      qk_norm_eps        queries and keys are divided by their root mean square after the rotation (None: not);
+      scale              the scores' factor;
+      sinks              one learned logit per query head that joins every softmax sum and has no value;
+      value_mix          'source': the values of the step's tokens are left for later layers under `value_mix_key`;
+                         'mix': v <- (1 - vmix) v + vmix (those values), before the cache is written;
+      output_gate        the heads are multiplied by sigmoid(gate projection of the mixer's input) before the output
+                         projection.
+
+    q, k, v and the gate are one product."""
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, scale: float,
+                 sinks: bool = False, qk_norm_eps: float | None = None, output_gate: bool = False,
+                 value_mix: str | None = None, value_mix_key: str = "values", window: int | None = None,
+                 position_encoding: PartSpec | None = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"sink_attention: {num_heads} heads do not split over {num_kv_heads} kv heads")
+        if value_mix not in (None, "source", "mix"):
+            raise ValueError(f"sink_attention: value_mix is None, 'source' or 'mix', not {value_mix!r}")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.key_dim, self.value_dim, self.scale = int(key_dim), int(value_dim), float(scale)
+        self.sinks, self.output_gate = bool(sinks), bool(output_gate)
+        self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
+        self.value_mix, self.value_mix_key = value_mix, str(value_mix_key)
+        self.window = int(window) if window else None
+        self.position_encoding = (POSITION_ENCODINGS.build(position_encoding.kind, **position_encoding.params)
+                                  if position_encoding is not None else None)
+        if self.position_encoding is not None and not hasattr(self.position_encoding, "frequencies"):
+            raise ValueError("sink_attention: the position encoding must give frequencies() (partial_rope)")
+        self.in_proj = self.o_proj = self.sink = self.vmix = None
+
+    def param_specs(self):
+        D, H, K, dk, dv = self.hidden_size, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        specs = {"q_proj": ParamSpec((H * dk, D)), "k_proj": ParamSpec((K * dk, D)), "v_proj": ParamSpec((K * dv, D)),
+                 "o_proj": ParamSpec((D, H * dv))}
+        if self.output_gate:
+            specs["gate_proj"] = ParamSpec((H * dv, D))
+        if self.sinks:
+            specs["sink"] = ParamSpec((H,), role="vector", init="norm")
+        if self.value_mix is not None:   # (a source stores the factor too and leaves it unused)
+            specs["vmix"] = ParamSpec((), role="vector", init="norm")
+        return specs
+
+    def load(self, tensors):
+        rows = [tensors["q_proj"], tensors["k_proj"], tensors["v_proj"]]
+        if self.output_gate:
+            rows.append(tensors["gate_proj"])
+        self.in_proj = as_product_weight(torch.cat(rows, dim=0).contiguous())
+        self.o_proj = as_product_weight(tensors["o_proj"])
+        self.sink = tensors["sink"].contiguous() if self.sinks else None
+        self.vmix = tensors["vmix"].reshape(1).contiguous() if self.value_mix is not None else None
+        if self.position_encoding is not None:
+            self.position_encoding.to_device(tensors["o_proj"].device)
+
+    def cache_need(self):
+        return PagedKVNeed(self.num_kv_heads, self.key_dim, self.window, self.value_dim)
+
+    def forward(self, x, ctx, cache, defer_sum=False):
+        H, K, dk, dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        group = ctx.groups[cache.group_id]
+        proj = ops.gemm(x, self.in_proj)
+        inv_freq, rot_dims = self.position_encoding.frequencies() if self.position_encoding is not None else (None, 0)
+        v_at = (H + K) * dk
+        v_first = None
+        if self.value_mix == "mix":
+            v_first = ctx.carry.get(self.value_mix_key)
+            if v_first is None:
+                raise RuntimeError(f"sink_attention: no earlier layer of the step has left {self.value_mix_key!r}")
+        write = cache.write
+        ops.qk_norm_rope_cache_write(proj, ctx.positions, inv_freq, rot_dims, self.qk_norm_eps, H, K, dk, dv,
+                                     v_first=v_first, v_mix=self.vmix if v_first is not None else None,
+                                     slot_mapping=group.slot_mapping if write else None,
+                                     k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
+        if self.value_mix == "source":
+            ctx.carry[self.value_mix_key] = proj[:, v_at:v_at + K * dv]
+        o = ops.paged_attention_sink(proj, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq, ctx.positions,
+                                     H, scale=self.scale, sinks=self.sink, window=self.window)
+        if self.output_gate:
+            g_at = v_at + K * dv
+            ops.gated_heads(o, proj[:, g_at:g_at + H * dv], H, dv, kind=ops.GATE_SIGMOID, out=o)
+        return ops.gemm(o, self.o_proj, defer_sum=defer_sum)

@@ -72,23 +72,28 @@ class PagedNeed:
 @dataclasses.dataclass(frozen=True)
 class PagedKVNeed(PagedNeed):
     """A mixer that keeps keys and values of earlier tokens: per token `num_kv_heads * head_dim`
-    keys and as many values; `window` None keeps all tokens, else only the last `window`.
+    keys and as many values (or `num_kv_heads * value_dim`, where the values have a size of their own); `window`
+    None keeps all tokens, else only the last `window`.
 
     Pages in the layout that the attention kernels read: keys "k" [page, kv head, page_size, head_dim] (inside a
     page in 16-key x 32-dimension operand blocks when the sizes allow: simply_amd/kernels/packing.py), values "v"
-    transposed [page, kv head, head_dim, page_size], so that the keys of a page are contiguous for each dimension."""
+    transposed [page, kv head, value size, page_size], so that the keys of a page are contiguous for each dimension."""
 
     num_kv_heads: int
     head_dim: int
     window: int | None = None
+    #: size of a value; None: the key size
+    value_dim: int | None = None
 
     def page_tensors(self, num_pages, page_size, dtype, device, fill):
         K, hd = self.num_kv_heads, self.head_dim
+        vd = hd if self.value_dim is None else self.value_dim
         return {"k": torch.full((num_pages, K, page_size, hd), fill, dtype=dtype, device=device),
-                "v": torch.full((num_pages, K, hd, page_size), fill, dtype=dtype, device=device)}
+                "v": torch.full((num_pages, K, vd, page_size), fill, dtype=dtype, device=device)}
 
     def bytes_per_token(self, esize):
-        return 2 * self.num_kv_heads * self.head_dim * esize
+        vd = self.head_dim if self.value_dim is None else self.value_dim
+        return self.num_kv_heads * (self.head_dim + vd) * esize
 
 
 @dataclasses.dataclass(frozen=True)

@@ -64,3 +64,35 @@ class SandwichBlock(Block):
         y = self.feed_forward.forward(give(self.feed_forward, x), ctx)
         h = x.settle()
         return h, PendingNorm(h, y, n["post_ffn"], next_norm, ctx.dtype)
+
+
+@BLOCKS.register("post_norm")
+class PostNormBlock(Block):
+    """h += post_mixer(mixer(h));  h += post_ffn(ffn(h)): the parts read the residual stream itself (in the
+    activation type), only what they return is normed.  A layer may have no feed-forward; then the second step is
+    left out.  A constant that scales what is added (a residual multiplier) is the norms' own factor.  Norms: 'input'
+    (what stands in front of both parts: usually the norm that is none), 'post_mixer', and 'post_ffn' if there is a
+    feed-forward."""
+
+    def __init__(self, mixer, feed_forward, norms):
+        super().__init__(mixer, feed_forward, norms)
+        wanted = ("input", "post_mixer") + (("post_ffn",) if feed_forward is not None else ())
+        missing = [n for n in wanted if n not in self.norms]
+        if missing:
+            raise ValueError(f"post_norm block: norms missing: {missing}")
+
+    def first_norm(self):
+        return self.norms["input"]
+
+    def forward(self, h, ctx, cache, normed, next_norm):
+        n = self.norms
+        if isinstance(normed, PendingNorm):
+            normed, h = normed.materialize(), normed.residual
+        if normed is None:
+            normed = n["input"].forward(h, ctx.dtype)
+        y = self.mixer.forward(normed, ctx, cache)
+        if self.feed_forward is None:
+            return h, n["post_mixer"].add_into(h, y, next_norm, ctx.dtype)
+        normed = n["post_mixer"].add_into(h, y, n["input"], ctx.dtype)
+        y = self.feed_forward.forward(normed, ctx)
+        return h, n["post_ffn"].add_into(h, y, next_norm, ctx.dtype)

@@ -15,6 +15,31 @@ ACTIVATIONS.register("silu", ops.ACT_SILU)
 ACTIVATIONS.register("squared_relu", ops.ACT_SQUARED_RELU)
 
 
+@FEED_FORWARDS.register("dense")
+class Dense(FeedForward):
+    """down(act(up(x))): one factor, no gate (simply/model_lib.py:643-730 with use_gated_activation_in_ffn=False)."""
+
+    defers_sum = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "squared_relu"):
+        self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
+        self.activation = activation
+        self.activation_code = int(ACTIVATIONS.get(activation))
+        self.up_proj = self.down_proj = None
+
+    def param_specs(self):
+        D, F = self.hidden_size, self.intermediate_size
+        return {"up_proj": ParamSpec((F, D)), "down_proj": ParamSpec((D, F))}
+
+    def load(self, tensors):
+        self.up_proj = as_product_weight(tensors["up_proj"])
+        self.down_proj = as_product_weight(tensors["down_proj"])
+
+    def forward(self, x: torch.Tensor, ctx=None, defer_sum=False) -> torch.Tensor:
+        z = ops.activation_(ops.gemm(x, self.up_proj), self.activation_code)
+        return ops.gemm(z, self.down_proj, defer_sum=defer_sum)
+
+
 @FEED_FORWARDS.register("gated_dense")
 class GatedDense(FeedForward):
     accepts_pending = True

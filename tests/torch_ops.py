@@ -201,6 +201,153 @@ def decode_attention_takes(q, k_pages, num_heads, max_q_len):
     return False
 
 
+def paged_attention_sink(q, k_pages, v_pages, block_table, token_seq, positions, num_heads, *, scale=1.0, sinks=None,
+                         window=None, soft_cap=None, out=None):
+    T = q.shape[0]
+    _, Kh, P, dk = k_pages.shape
+    dv = v_pages.shape[2]
+    k_pages = stored_keys_as_rows(k_pages)
+    H = num_heads
+    G = H // Kh
+    res = torch.empty((T, H * dv), dtype=q.dtype, device=q.device)
+    for t in range(T):
+        pos = int(positions[t])
+        lo = max(pos - window + 1, 0) if window else 0
+        keys = torch.arange(lo, pos + 1, device=q.device)
+        pages = block_table[int(token_seq[t]), keys // P].long()
+        assert (pages >= 0).all(), "attention reads a key that has no page"
+        k = _f(k_pages[pages, :, keys % P])          # [n, Kh, dk]
+        v = _f(v_pages[pages, :, :, keys % P])       # [n, Kh, dv]
+        qt = _f(q[t, :H * dk]).reshape(Kh, G, dk)
+        s = torch.einsum("kgd,nkd->kgn", qt, k) * scale
+        if soft_cap:
+            s = soft_cap * torch.tanh(s / soft_cap)
+        if sinks is not None:
+            s = torch.cat([s, _f(sinks).reshape(Kh, G, 1)], dim=-1)
+        p = torch.softmax(s, -1)[..., :len(keys)]
+        res[t] = torch.einsum("kgn,nkd->kgd", p, v).reshape(H * dv).to(q.dtype)
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
+
+
+def residual_add_norm(y, residual, *, weight=None, eps=0.0, plus_one=False, mult=1.0, out_dtype=None, out=None):
+    if hasattr(y, "materialize"):
+        y = y.materialize()
+    if y is not None:
+        v = _f(y)
+        if weight is not None:
+            v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * (_f(weight) + (1.0 if plus_one else 0.0))
+        residual.copy_((_f(residual) + mult * v).to(torch.float32))
+    if out is None and out_dtype is None:
+        return None
+    r = residual.to(out_dtype or out.dtype)
+    if out is not None:
+        out.copy_(r)
+        return out
+    return r
+
+
+GATE_SIGMOID, GATE_SILU = 0, 1
+
+
+def gated_heads(x, gate, num_heads, size, *, kind, weight=None, eps=0.0, out_dtype=None, out=None):
+    T = x.shape[0]
+    v = _f(x).reshape(T, num_heads, size)
+    if weight is not None:
+        v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * _f(weight)
+    g = _f(gate).reshape(T, num_heads, size)
+    g = torch.sigmoid(g) if kind == GATE_SIGMOID else g * torch.sigmoid(g)
+    r = (v * g).reshape(T, num_heads * size).to(out_dtype or (out.dtype if out is not None else x.dtype))
+    if out is not None:
+        out.copy_(r)
+        return out
+    return r
+
+
+def activation_(x, activation):
+    x.copy_(ACTIVATIONS[activation](_f(x)).to(x.dtype))
+    return x
+
+
+def qk_norm_rope_cache_write(proj, positions, inv_freq, rot_dims, eps, num_heads, num_kv_heads, key_dim, value_dim, *,
+                             v_first=None, v_mix=None, slot_mapping=None, k_pages=None, v_pages=None):
+    T = proj.shape[0]
+    H, K, dk, dv = num_heads, num_kv_heads, key_dim, value_dim
+    qk = _f(proj[:, :(H + K) * dk]).reshape(T, H + K, dk).clone()
+    if rot_dims:
+        half = rot_dims // 2
+        ang = (positions.to(torch.float32)[:, None] * inv_freq.to(torch.float32)[None, :]).to(qk.dtype)[:, None, :]
+        s, c = torch.sin(ang), torch.cos(ang)
+        a, b = qk[..., :half].clone(), qk[..., half:rot_dims].clone()
+        qk[..., :half] = a * c - b * s
+        qk[..., half:rot_dims] = b * c + a * s
+    if eps is not None:
+        qk = qk / torch.sqrt((qk * qk).mean(-1, keepdim=True) + eps)
+    proj[:, :H * dk] = qk[:, :H].reshape(T, H * dk).to(proj.dtype)
+    if k_pages is None:
+        return proj
+    P = k_pages.shape[2]
+    v = _f(proj[:, (H + K) * dk:(H + K) * dk + K * dv])
+    if v_first is not None:
+        lam = _f(v_mix).reshape(())
+        v = (1.0 - lam) * v + lam * _f(v_first)
+    page, off = (slot_mapping[:T] // P).long(), (slot_mapping[:T] % P).long()
+    krows = stored_keys_as_rows(k_pages)
+    krows[page, :, off] = qk[:, H:].to(k_pages.dtype)
+    k_pages.copy_(rows_as_stored_keys(krows))
+    v_pages[page, :, :, off] = v.reshape(T, K, dv).to(v_pages.dtype)
+    return proj
+
+
+def short_conv_silu(x, taps, tails, seq_meta, num_seqs, max_q_len, *, update_tails=True, out=None):
+    T, C = x.shape
+    n = taps.shape[1]
+    y = torch.empty((T, C), dtype=torch.float32, device=x.device) if out is None else out
+    w = _f(taps)
+    for slot, first, count, _ in seq_meta[:num_seqs].tolist():
+        old = _f(tails[slot, :(n - 1) * C]).reshape(n - 1, C)
+        xs = torch.cat([old, _f(x[first:first + count])], dim=0)
+        acc = sum(xs[j:j + count] * w[:, j][None, :] for j in range(n))
+        y[first:first + count] = (acc * torch.sigmoid(acc)).to(torch.float32)
+        if update_tails and n > 1:
+            tails[slot, :(n - 1) * C] = xs[count:].reshape(-1).to(torch.float32)
+    return y
+
+
+def delta_prepare(qkv, ab, a_log, dt_bias, num_heads, num_qk_heads, key_dim):
+    T, C = qkv.shape
+    H, G, dk = num_heads, num_qk_heads, key_dim
+    qk = _f(qkv[:, :2 * G * dk]).reshape(T, 2 * G, dk)
+    qk = qk / torch.sqrt((qk * qk).sum(-1, keepdim=True) + 1e-6)
+    qk[:, :G] = qk[:, :G] * dk ** -0.5
+    qkv[:, :2 * G * dk] = qk.reshape(T, -1).to(torch.float32)
+    a, b = _f(ab[:, :H]), _f(ab[:, H:2 * H])
+    g = torch.exp(-torch.exp(_f(a_log)) * torch.nn.functional.softplus(a + _f(dt_bias), threshold=30.0))
+    return torch.cat([torch.sigmoid(b), g], dim=1).to(torch.float32)
+
+
+def delta_rule(qkv, gates, state, seq_meta, num_seqs, num_heads, num_qk_heads, key_dim, value_dim):
+    T, C = qkv.shape
+    H, G, dk, dv = num_heads, num_qk_heads, key_dim, value_dim
+    out = torch.empty((T, H * dv), dtype=torch.float32, device=qkv.device)
+    x, gt = _f(qkv), _f(gates)
+    for slot, first, count, _ in seq_meta[:num_seqs].tolist():
+        S = _f(state[slot, :H * dk * dv]).reshape(H, dk, dv).clone()
+        for t in range(first, first + count):
+            for h in range(H):
+                j = h // (H // G)
+                q, k = x[t, j * dk:(j + 1) * dk], x[t, (G + j) * dk:(G + j + 1) * dk]
+                v = x[t, 2 * G * dk + h * dv:2 * G * dk + (h + 1) * dv]
+                S[h] = gt[t, H + h] * S[h]
+                u = gt[t, h] * (v - S[h].T @ k)
+                S[h] = S[h] + torch.outer(k, u)
+                out[t, h * dv:(h + 1) * dv] = (S[h].T @ q).to(torch.float32)
+        state[slot, :H * dk * dv] = S.reshape(-1).to(torch.float32)
+    return out
+
+
 # ---- sampling: the same counter-based generator as the kernel, in integer arithmetic
 
 
