@@ -1,0 +1,117 @@
+"""Zenuzen on the GPU: every kernel against the plain implementation's function for its mechanism, the mixers as
+parts with a cache or a state of their own, and the engine (whole prompts, token-by-token decoding, portions down to
+two tokens, unequal requests together in a tight pool, long decoding, recorded decode steps, greedy generation
+through the scheduler) against the plain implementation, in 32-bit and in bfloat16."""
+import pytest
+import torch
+
+import plain_zenuzen as plain
+import zenuzen_cases as cases
+import zenuzen_mechanisms as mech
+from simply_amd.engine import StepEntry
+from simply_amd.kernels import ops
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(autouse=True)
+def _lib(gpu_lib):
+    return gpu_lib
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("body", [mech.residual_add_norm, mech.gated_heads, mech.activation,
+                                  mech.partial_rotary_norm_and_pages, mech.sink_attention_far_key, mech.short_convolution])
+def test_kernel(body, dtype):
+    body(ops, DEV, dtype)
+
+
+def test_partial_rotary_into_tiled_pages():
+    """Pages of 16 keys of a size that is a multiple of 32 are stored in operand blocks: the same test, that layout."""
+    mech.partial_rotary_norm_and_pages(ops, DEV, torch.bfloat16, page_size=16)
+
+
+def test_recurrence_kernel():
+    mech.delta_rule_steps(ops, DEV)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_part(dtype):
+    mech.attention_part(DEV, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_delta_part(dtype):
+    mech.delta_part(DEV, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["mixed", "only_delta", "only_attention", "aligned"])
+def test_cuts_match_plain(tmp_path, name, dtype):
+    cases.cuts_match_plain(tmp_path, DEV, name, dtype, length=45 if name != "aligned" else 70)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["mixed", "only_delta", "aligned"])
+def test_batches_match_alone(tmp_path, name, dtype):
+    cases.batches_match_alone(tmp_path, DEV, name, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding(tmp_path, dtype):
+    cases.long_decoding(tmp_path, DEV, "mixed", dtype, steps=150, page_size=16)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_decode_steps(tmp_path, dtype):
+    """Decode-only steps are recorded in a HIP graph and replayed: three requests decode together for 40 steps, and
+    each step's logits are those of the same step run eagerly by a second engine (states advance exactly once)."""
+    d = cases.write_model("mixed", str(tmp_path / "m"))
+    V = plain.load(d)[1]["vocab"]
+    prompts = {r: cases.random_tokens(n, V, 70 + n) for r, n in (("a", 9), ("b", 3), ("c", 14))}
+    follow = {r: cases.random_tokens(40, V, 90 + len(p)) for r, p in prompts.items()}
+    engines = [cases.make_executor(d, DEV, dtype, page_size=4, num_pages=64, batch=4, max_len=64, graphs=g)
+               for g in (True, False)]
+    for ex in engines:
+        for r, p in prompts.items():
+            ex.add_request(r)
+        ex.step([StepEntry(r, p, []) for r, p in prompts.items()])
+    for k in range(40):
+        outs = [ex.step([StepEntry(r, [follow[r][k]], [0]) for r in prompts]).clone() for ex in engines]
+        torch.testing.assert_close(outs[0], outs[1], rtol=0, atol=0)
+
+
+def test_greedy_generation(tmp_path):
+    cases.greedy_generation(tmp_path, DEV, "mixed", "float32")
+
+
+def test_trace_replay_child_process(tmp_path):
+    """bin/trace_run as a user starts it: a folder, steps on standard input, logits in files."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+
+    d = cases.write_model("mixed", str(tmp_path / "m"), dtype=torch.bfloat16)
+    w, cfg = plain.load(d)
+    tokens = cases.random_tokens(30, cfg["vocab"], 5)
+    want = plain.forward(w, cfg, tokens)
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": tokens[:17], "want": [0, 16]}], "end": []},
+             {"step": 1, "entries": [{"id": "x", "tokens": tokens[17:19], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "x", "tokens": tokens[19:], "want": [10]}], "end": ["x"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", d, "--dtype", "float32", "--out", str(out),
+                        "--max-tokens", "64"], input="\n".join(json.dumps(s) for s in steps) + "\n", text=True,
+                       capture_output=True, timeout=600)
+    assert r.returncode == 0, r.stderr
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
+    assert not (out / "1.f32").exists()
+    got0 = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(2, -1))
+    got2 = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(1, -1))
+    assert cases.rel_error(got0, want[[0, 16]]) <= cases.BOUND["float32"]
+    assert cases.rel_error(got2, want[[29]]) <= cases.BOUND["float32"]

@@ -1,0 +1,125 @@
+"""Zenuzen on the CPU: configuration and weights, every mechanism's plain torch reference against the plain
+implementation's function, and the framework's host logic (model, parts, cache and state manager, step function,
+scheduler) with the kernels replaced by those references."""
+import json
+
+import pytest
+import torch
+
+import plain_zenuzen as plain
+import torch_ops
+import zenuzen_cases as cases
+import zenuzen_mechanisms as mech
+from simply_amd.config import ConfigError, ZenuzenConfig, config_from_dict, load_config
+from simply_amd.models import DecoderModel
+from simply_amd.weights import WeightsError
+
+CPU = "cpu"
+
+
+# ------------------------------------------------------------------ configuration, registry, weights
+def test_config_round_trip_and_spec():
+    cfg = config_from_dict(cases.MIXED)
+    assert isinstance(cfg, ZenuzenConfig) and config_from_dict(cfg.to_dict()) == cfg
+    spec = cfg.model_spec()
+    kinds = [l.mixer.kind for l in spec.layers]
+    assert kinds == ["sink_attention", "gated_delta", "sink_attention", "gated_delta", "sink_attention", "gated_delta"]
+    # the first layer that mixes values is their source, later ones mix, others neither
+    assert [l.mixer.params.get("value_mix") for l in spec.layers if l.mixer.kind == "sink_attention"] == ["source", "mix", None]
+    assert [l.feed_forward is not None for l in spec.layers] == [False, True, True, False, False, False]
+    assert all(l.norms["post_mixer"].params["mult"] == 0.55 for l in spec.layers)
+    model = DecoderModel(spec)
+    names = model.expected_tensors()
+    assert names["l0.mix.vmix"].shape == () and names["l1.mix.q.conv"].shape == (60, 3)
+    assert "l0.norm2" not in names and "l1.norm2" in names and "l4.mix.vmix" not in names
+    needs = [n for n, _ in model.cache_needs()]
+    assert needs[0].value_dim == 40 and needs[0].head_dim == 24
+    assert needs[1].shape == (3 * 20 * 24 + 2 * (2 * 3 * 20 + 3 * 24),)
+
+
+@pytest.mark.parametrize("change, message", [
+    (lambda d: d["layers"][0].update(type="conv"), "unknown layer type"),
+    (lambda d: d["layers"][0]["mixer"].pop("scale"), "scale"),
+    (lambda d: d["layers"][0]["mixer"].update(heads=3, kv_heads=2), "multiple"),
+    (lambda d: d["layers"][0]["mixer"]["rot"].update(dims=7), "even"),
+    (lambda d: d["layers"][1]["mixer"].update(conv=0), "conv"),
+    (lambda d: d["layers"][1]["mlp"].update(kind="routed"), "unknown kind"),
+    (lambda d: d["layers"][2]["mixer"].update(vdim=8), "agree"),
+    (lambda d: d.pop("residual_mult"), "residual_mult"),
+    (lambda d: d["norm"].pop("eps"), "eps"),
+])
+def test_config_errors(change, message):
+    d = json.loads(json.dumps(cases.MIXED))
+    change(d)
+    with pytest.raises(ConfigError, match=message):
+        config_from_dict(d)
+
+
+def test_folder_round_trip_and_missing_tensor(tmp_path):
+    d = cases.write_model("mixed", str(tmp_path / "m"))
+    assert load_config(d) == config_from_dict(cases.MIXED)
+    from safetensors.torch import load_file, save_file
+    from simply_amd.engine.loading import load_model
+
+    tensors = load_file(f"{d}/model.safetensors")
+    tensors.pop("l2.mix.sink")
+    tensors["l2.mix.bias"] = torch.zeros(3)
+    save_file(tensors, f"{d}/model.safetensors")
+    with pytest.raises(WeightsError) as e:
+        load_model(d, torch.float32, "cpu")
+    assert e.value.missing == ["l2.mix.sink"] and e.value.unexpected == ["l2.mix.bias"]
+
+
+# ------------------------------------------------------------------ the references of the kernels, one by one
+@pytest.mark.parametrize("body", [mech.residual_add_norm, mech.gated_heads, mech.activation,
+                                  mech.partial_rotary_norm_and_pages, mech.sink_attention_far_key, mech.short_convolution])
+def test_reference_of_a_kernel(body):
+    body(torch_ops, CPU, torch.float32)
+
+
+def test_reference_of_the_recurrence():
+    mech.delta_rule_steps(torch_ops, CPU)
+
+
+def test_attention_part(cpu_ops):
+    mech.attention_part(CPU, torch.float32)
+
+
+def test_delta_part(cpu_ops):
+    mech.delta_part(CPU, torch.float32)
+
+
+# ------------------------------------------------------------------ the engine's host logic
+@pytest.mark.parametrize("name", ["mixed", "only_delta", "only_attention"])
+def test_cuts_match_plain(tmp_path, cpu_ops, name):
+    cases.cuts_match_plain(tmp_path, CPU, name)
+
+
+@pytest.mark.parametrize("name", ["mixed", "only_delta"])
+def test_batches_match_alone(tmp_path, cpu_ops, name):
+    cases.batches_match_alone(tmp_path, CPU, name)
+
+
+def test_long_decoding(tmp_path, cpu_ops):
+    cases.long_decoding(tmp_path, CPU, "mixed", steps=70, page_size=4)
+
+
+def test_greedy_generation(tmp_path, cpu_ops):
+    cases.greedy_generation(tmp_path, CPU)
+
+
+def test_plain_portions_of_the_recurrence_and_the_convolution():
+    """The plain implementation itself: carried over a cut, the recurrence and the convolution give what they give
+    in one piece (the state and the last inputs are all that a later portion needs)."""
+    T, H, dk, dv = 12, 2, 5, 7
+    q, k, v = mech.rand((T, H, dk), 1), mech.rand((T, H, dk), 2), mech.rand((T, H, dv), 3)
+    beta, g = torch.sigmoid(mech.rand((T, H), 4)), torch.sigmoid(mech.rand((T, H), 5))
+    whole, S = plain.delta_recurrence(q, k, v, beta, g)
+    a, Sa = plain.delta_recurrence(q[:5], k[:5], v[:5], beta[:5], g[:5])
+    b, Sb = plain.delta_recurrence(q[5:], k[5:], v[5:], beta[5:], g[5:], Sa)
+    torch.testing.assert_close(torch.cat([a, b]), whole)
+    torch.testing.assert_close(Sb, S)
+    x, taps = mech.rand((9, 4), 6), mech.rand((4, 3), 7)
+    y = plain.causal_conv(x, taps)
+    torch.testing.assert_close(y[0], x[0] * taps[:, 2])
+    torch.testing.assert_close(y[4], x[4] * taps[:, 2] + x[3] * taps[:, 1] + x[2] * taps[:, 0])
