@@ -343,6 +343,111 @@ def measure_ceilings():
     return out
 
 
+# --only zenuzen: layer sizes that resemble a real model's, for the Zenuzen design (three layers with the gated
+# delta rule to one with attention, a dense feed-forward in every layer) and, beside it, Gemma 2 layers of equal width,
+# depth, head count and head size whose gated feed-forward has as many parameters
+ZENUZEN_SIZES = {
+    "small": dict(width=1024, heads=8, kv_heads=2, dim=128, ff=4096, vocab=32768),
+    "medium": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=8192, vocab=32768),
+    "large": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=14336, vocab=32768),
+}
+
+
+def zenuzen_config(size: dict, layers: int) -> dict:
+    W, H, K, d = size["width"], size["heads"], size["kv_heads"], size["dim"]
+    out = []
+    for i in range(layers):
+        mlp = {"kind": "dense", "ff": size["ff"]}
+        if i % 4 == 3:
+            out.append({"type": "attention", "mlp": mlp,
+                        "mixer": {"heads": H, "kv_heads": K, "dim": d, "vdim": d, "scale": d ** -0.5, "v_mix": True,
+                                  "rot": {"dims": d // 2, "base": 1000000.0}}})
+        else:
+            out.append({"type": "delta", "mlp": mlp,
+                        "mixer": {"heads": H, "kv_heads": H // 2, "dim": d, "vdim": d, "conv": 4}})
+    return {"architecture": "Zenuzen", "vocab": size["vocab"], "width": W, "residual_mult": 0.7, "norm": {"eps": 1e-5},
+            "layers": out}
+
+
+def gemma_of_equal_size(size: dict, layers: int) -> dict:
+    ff = (2 * size["ff"] // 3 + 255) // 256 * 256    # three matrices instead of two
+    return dict(GEMMA2_2B, hidden_size=size["width"], num_hidden_layers=layers, num_attention_heads=size["heads"],
+                num_key_value_heads=size["kv_heads"], head_dim=size["dim"], intermediate_size=ff,
+                vocab_size=size["vocab"], query_pre_attn_scalar=size["dim"], sliding_window=None)
+
+
+def run_executor_bench(model, vocab, prefill_tokens, batch, context, steps, warmup, page_size, dtype):
+    """Through the step function alone (no scheduler, no sampler): seconds for a prompt of `prefill_tokens` in one
+    step with the logits of its last token, and seconds per decode step of `batch` requests that hold `context`
+    tokens each (recorded steps, the host preparing every step)."""
+    import torch
+    from simply_amd.config import EngineConfig
+    from simply_amd.engine import Executor, StepEntry
+
+    g = torch.Generator().manual_seed(3)
+    max_len = max(prefill_tokens, context + steps + warmup) + 16
+    cfg = EngineConfig(activation_dtype=dtype, page_size=page_size, batch_size=batch, max_seq_len=max_len,
+                       max_num_issue_tokens=max(prefill_tokens, 2048),
+                       total_num_pages=-(-max_len // page_size) * batch + 8, use_graphs=True)
+    ex = Executor(model, cfg)
+    times = []
+    for rep in range(4):
+        prompt = torch.randint(0, vocab, (prefill_tokens,), generator=g).tolist()
+        ex.add_request("p")
+        sync()
+        t0 = time.perf_counter()
+        ex.step([StepEntry("p", prompt, [prefill_tokens - 1])])
+        sync()
+        times.append(time.perf_counter() - t0)
+        ex.finish_request("p")
+    prefill = min(times[1:])
+    rids = [f"d{i}" for i in range(batch)]
+    for r in rids:
+        ex.add_request(r)
+        done = 0
+        while done < context:
+            n = min(2048, context - done)
+            ex.step([StepEntry(r, torch.randint(0, vocab, (n,), generator=g).tolist(), [])])
+            done += n
+    def decode(k):
+        for _ in range(k):
+            toks = torch.randint(0, vocab, (batch,), generator=g).tolist()
+            ex.step([StepEntry(r, [t], [0]) for r, t in zip(rids, toks)])
+    decode(warmup)
+    sync()
+    t0 = time.perf_counter()
+    decode(steps)
+    sync()
+    dt = (time.perf_counter() - t0) / steps
+    del ex
+    torch.cuda.empty_cache()
+    return prefill, dt
+
+
+def run_zenuzen(args):
+    import torch
+    from simply_amd.config import config_from_dict
+    from simply_amd.engine.loading import random_model
+
+    tdtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    layers = args.layers or 8
+    for name in args.sizes.split(","):
+        size = ZENUZEN_SIZES[name]
+        for label, d in (("zenuzen", zenuzen_config(size, layers)), ("gemma2-equal-size", gemma_of_equal_size(size, layers))):
+            cfg = config_from_dict(d)
+            model = random_model(cfg, 0, tdtype, torch.device("cuda:0"), std=0.02)
+            pt, dt = run_executor_bench(model, size["vocab"], args.prefill_tokens, args.batch, args.context, args.steps,
+                                        args.warmup, args.page_size, args.dtype)
+            print(json.dumps({"metric": "prefill and decode tokens/s through the step function", "model": label,
+                              "size": name, "width": size["width"], "layers": layers,
+                              "prefill_tokens": args.prefill_tokens, "prefill_tokens_per_s": round(args.prefill_tokens / pt, 1),
+                              "prefill_ms": round(pt * 1e3, 3), "batch": args.batch, "context": args.context,
+                              "decode_tokens_per_s": round(args.batch / dt, 1), "decode_ms_per_step": round(dt * 1e3, 3),
+                              "dtype": args.dtype, "data": "synthetic"}), flush=True)
+            del model
+            torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -358,13 +463,15 @@ def main():
     ap.add_argument("--batches", default="1,8,32,64", help="--only decode-grid: the batch sizes")
     ap.add_argument("--contexts", default="1024,4096,8192", help="--only decode-grid: the context lengths")
     ap.add_argument("--only", default="all", choices=["all", "decode", "decode-grid", "prefill", "prefill-chunked", "products",
-                                                      "gated-products", "ceilings"],
+                                                      "gated-products", "ceilings", "zenuzen"],
                     help="measure one part alone (for profiles); the line then holds that part only.  products / "
                          "gated-products: the sweep of the product kernels over rows and weight sizes; ceilings: "
                          "what the GPU itself reaches in reading HBM and in bfloat16 MFMA instructions")
     ap.add_argument("--latency-steps", type=int, default=100,
                     help="decode steps run one at a time after the timed ones, for the p50 and p99 of a step's latency")
     ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="layer sizes: Gemma 2 2B (the default), 9B, 27B")
+    ap.add_argument("--sizes", default="small,medium,large",
+                    help="--only zenuzen: which of the layer sizes small, medium, large (8 layers each, or --layers)")
     ap.add_argument("--requests", type=int, default=0,
                     help="instead of timed decode steps: a workload of this many requests through the scheduler")
     ap.add_argument("--prompt-min", type=int, default=128)
@@ -387,6 +494,9 @@ def main():
         return
     if args.only in ("products", "gated-products"):
         run_products("gated" if args.only == "gated-products" else "plain")
+        return
+    if args.only == "zenuzen":
+        run_zenuzen(args)
         return
     d = dict(GEMMA2_2B, **SHAPES[args.shape])
     full_layers = d["num_hidden_layers"]

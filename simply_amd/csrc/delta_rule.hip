@@ -103,35 +103,46 @@ __global__ __launch_bounds__(kWave) void delta_prepare_kernel(float* __restrict_
   }
 }
 
-// The recurrence.  A workgroup of 256 threads takes 64 columns of one head's state for one request: four lanes
-// share a column, lane `part` of them holding rows part, part + 4, ... of it in registers (DK / 4 of them).  The
-// step's q and k of kRuleTokens tokens at a time go through LDS.  Columns are independent of each other, rows are
-// summed within a lane in increasing order and then across the four lanes in a fixed order.
+// The recurrence.  A workgroup of 256 threads takes 256 / LPC columns of one head's state for one request: LPC lanes
+// (4 or 16, neighbours in a row of 16 lanes) share a column, lane `part` of them holding rows part, part + LPC, ...
+// of it in registers (DK / LPC of them).  The step's q, k and v of kRuleTokens tokens at a time go through LDS.
+// Columns are independent of each other; a column's sums run within a lane over its rows in increasing order, in
+// four partial sums that are added in a fixed order, then across the lanes by data-parallel primitives in a fixed
+// order: nothing depends on how the tokens are cut into steps or on the batch.  The chain of dependent operations
+// per token is what bounds a prompt's time (tokens follow one another): 16 lanes per column keep it short where a
+// column has 64 rows or more.
 constexpr int kRuleTokens = 16;
-__device__ __forceinline__ float quad_sum(float v) {
+template <int LPC>
+__device__ __forceinline__ float lanes_sum(float v) {
   v += lane_exchange<0xB1>(v);   // quad_perm [1, 0, 3, 2]
   v += lane_exchange<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  if (LPC == 16) {
+    v += lane_exchange<0x141>(v);  // row_half_mirror
+    v += lane_exchange<0x140>(v);  // row_mirror
+  }
   return v;
 }
 
-template <int DK>
+template <int DK, int LPC>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ qkv, int C, int G, int dk, int dv,
                                                          const float* __restrict__ gates, int H,
                                                          float* __restrict__ state, int64_t state_stride,
                                                          const int* __restrict__ seq_meta, float* __restrict__ out) {
-  constexpr int R = DK / 4;
-  __shared__ float qs[kRuleTokens][DK], ks[kRuleTokens][DK], vs[kRuleTokens][64], bg[kRuleTokens][2];
+  constexpr int R = DK / LPC, COLS = 256 / LPC;
+  static_assert(R % 4 == 0 || R < 4, "rows per lane come in fours");
+  constexpr int NACC = R < 4 ? 1 : 4;
+  __shared__ float qs[kRuleTokens][DK], ks[kRuleTokens][DK], vs[kRuleTokens][COLS], bg[kRuleTokens][2];
   const int* meta = seq_meta + 4 * blockIdx.x;
   const int slot = meta[0], first = meta[1], count = meta[2];
   const int h = blockIdx.y, tid = threadIdx.x;
-  const int col = blockIdx.z * 64 + tid / 4, part = tid % 4;
+  const int col = blockIdx.z * COLS + tid / LPC, part = tid % LPC;
   const bool live = col < dv;
   const int qk_head = h / (H / G);
   float* S = state + static_cast<size_t>(slot) * state_stride + static_cast<size_t>(h) * dk * dv;   // [dk][dv]
   float s[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int i = r * 4 + part;
+    const int i = r * LPC + part;
     s[r] = (live && i < dk) ? S[static_cast<size_t>(i) * dv + col] : 0.f;
   }
   const int v_at = 2 * G * dk + h * dv;
@@ -144,37 +155,48 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
       qs[j][i] = i < dk ? row[qk_head * dk + i] : 0.f;
       ks[j][i] = i < dk ? row[(G + qk_head) * dk + i] : 0.f;
     }
-    for (int idx = tid; idx < tn * 64; idx += 256) {
-      const int j = idx / 64, c = blockIdx.z * 64 + idx % 64;
-      vs[j][idx % 64] = c < dv ? qkv[static_cast<size_t>(first + t0 + j) * C + v_at + c] : 0.f;
+    for (int idx = tid; idx < tn * COLS; idx += 256) {
+      const int j = idx / COLS, c = blockIdx.z * COLS + idx % COLS;
+      vs[j][idx % COLS] = c < dv ? qkv[static_cast<size_t>(first + t0 + j) * C + v_at + c] : 0.f;
     }
     if (tid < 2 * tn) bg[tid / 2][tid % 2] = gates[static_cast<size_t>(first + t0 + tid / 2) * 2 * H + (tid % 2) * H + h];
     __syncthreads();
     for (int j = 0; j < tn; ++j) {
       const size_t t = static_cast<size_t>(first + t0 + j);
       const float beta = bg[j][0], g = bg[j][1];
-      const float v = vs[j][tid / 4];
-      float dot = 0.f;
+      const float v = vs[j][tid / LPC];
+      float kr[R], qr[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        kr[r] = ks[j][r * LPC + part];
+        qr[r] = qs[j][r * LPC + part];
+      }
+      float d[NACC];
+#pragma unroll
+      for (int a = 0; a < NACC; ++a) d[a] = 0.f;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         s[r] *= g;
-        dot = fmaf(s[r], ks[j][r * 4 + part], dot);
+        d[r % NACC] = fmaf(s[r], kr[r], d[r % NACC]);
       }
-      dot = quad_sum(dot);
+      float dot = NACC == 4 ? (d[0] + d[1]) + (d[2] + d[3]) : d[0];
+      dot = lanes_sum<LPC>(dot);
       const float u = beta * (v - dot);
-      float o = 0.f;
+#pragma unroll
+      for (int a = 0; a < NACC; ++a) d[a] = 0.f;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        s[r] = fmaf(ks[j][r * 4 + part], u, s[r]);
-        o = fmaf(s[r], qs[j][r * 4 + part], o);
+        s[r] = fmaf(kr[r], u, s[r]);
+        d[r % NACC] = fmaf(s[r], qr[r], d[r % NACC]);
       }
-      o = quad_sum(o);
+      float o = NACC == 4 ? (d[0] + d[1]) + (d[2] + d[3]) : d[0];
+      o = lanes_sum<LPC>(o);
       if (live && part == 0) out[t * (static_cast<size_t>(H) * dv) + static_cast<size_t>(h) * dv + col] = o;
     }
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int i = r * 4 + part;
+    const int i = r * LPC + part;
     if (live && i < dk) S[static_cast<size_t>(i) * dv + col] = s[r];
   }
 }
@@ -187,8 +209,8 @@ extern "C" int sa_short_conv_silu(const void* x, int x_dtype, int64_t x_stride, 
                                   int num_taps, float* tails, int64_t tail_stride, const int* seq_meta, int num_seqs,
                                   int max_q_len, float* y, int C, int update_tails, hipStream_t stream) {
   if (num_seqs == 0 || max_q_len == 0) return 0;
-  SA_REQUIRE(num_seqs > 0 && max_q_len > 0 && C > 0 && x != nullptr && taps != nullptr && tails != nullptr &&
-                 seq_meta != nullptr && y != nullptr,
+  SA_REQUIRE(num_seqs > 0 && max_q_len > 0 && C > 0 && x != nullptr && taps != nullptr &&
+                 (tails != nullptr || num_taps == 1) && seq_meta != nullptr && y != nullptr,
              "short_conv_silu: bad sizes S=%d q=%d C=%d", num_seqs, max_q_len, C);
   SA_REQUIRE(num_taps >= 1 && num_taps <= kMaxTaps, "short_conv_silu: 1 to %d taps, got %d", kMaxTaps, num_taps);
   SA_REQUIRE(x_stride >= C && tail_stride >= static_cast<int64_t>(num_taps - 1) * C,
@@ -226,14 +248,15 @@ extern "C" int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, con
   SA_REQUIRE(state_stride >= static_cast<int64_t>(H) * dk * dv, "delta_rule: the state rows are too short");
   SA_REQUIRE(qkv != nullptr && gates != nullptr && state != nullptr && seq_meta != nullptr && out != nullptr,
              "delta_rule: a null pointer");
-  SA_REQUIRE(H <= 65535 && (dv + 63) / 64 <= 65535, "delta_rule: too many heads or columns");
-  const dim3 grid(num_seqs, H, (dv + 63) / 64);
-#define SA_DELTA_RULE(DK) \
-  delta_rule_kernel<DK><<<grid, 256, 0, stream>>>(qkv, C, G, dk, dv, gates, H, state, state_stride, seq_meta, out)
-  if (dk <= 32) SA_DELTA_RULE(32);
-  else if (dk <= 64) SA_DELTA_RULE(64);
-  else if (dk <= 128) SA_DELTA_RULE(128);
-  else SA_DELTA_RULE(256);
+  SA_REQUIRE(H <= 65535 && dv <= 65535 * 16, "delta_rule: too many heads or columns");
+#define SA_DELTA_RULE(DK, LPC)                                                                                      \
+  delta_rule_kernel<DK, LPC><<<dim3(num_seqs, H, (dv + 256 / LPC - 1) / (256 / LPC)), 256, 0, stream>>>(             \
+      qkv, C, G, dk, dv, gates, H, state, state_stride, seq_meta, out)
+  if (dk <= 16) SA_DELTA_RULE(16, 4);
+  else if (dk <= 32) SA_DELTA_RULE(32, 4);
+  else if (dk <= 64) SA_DELTA_RULE(64, 16);
+  else if (dk <= 128) SA_DELTA_RULE(128, 16);
+  else SA_DELTA_RULE(256, 16);
 #undef SA_DELTA_RULE
   return check_launch("delta_rule");
 }
