@@ -242,7 +242,7 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
                            const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                            float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
-                           hipStream_t stream);
+                           hipStream_t stream, const float* sinks = nullptr);
 int paged_attention_prefill_group();  // units that one workgroup takes
 bool paged_attention_prefill_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q,
                                    int64_t out_stride, const void* out);
@@ -250,7 +250,7 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
                             const int* block_table, int table_stride, const int* units, int unit_begin, int unit_count,
                             void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                             float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
-                            hipStream_t stream);
+                            hipStream_t stream, const float* sinks = nullptr);
 bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* A, const void* W, const void* W2,
                      const void* C, int c_dtype, int epi, int packed);
 int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int act,
@@ -298,11 +298,11 @@ int sa_activation(void* x, int dtype, int64_t stride, int T, int N, int act, hip
 
 // Rows [H * dk queries | K * dk keys | K * dv values | ...] of a fused projection: queries and keys are rotated on
 // their first rot_dims dimensions (pairs (i, i + rot_dims / 2), angle position * inv_freq[i]) and then divided by
-// sqrt(mean(x^2) + eps) over the head (eps < 0: not); queries go back in place, keys into the key pages; values
+// sqrt(mean(x^2) + eps) over the head (eps < 0: not); queries, times q_mult, go back in place, keys into the key pages; values
 // become (1 - *lambda) v + *lambda v_first[t] (v_first null: stay) and go into the value pages
 // [num_pages, K, dv, page_size].  k_pages null: nothing is written.
 int sa_qk_norm_rope_cache_write(void* proj, int dtype, int64_t row_stride, const int* positions, const float* inv_freq,
-                                int rot_dims, float eps, const void* v_first, int64_t v_first_stride,
+                                int rot_dims, float eps, float q_mult, const void* v_first, int64_t v_first_stride,
                                 const void* lambda, int lambda_dtype, const int64_t* slot_mapping, void* k_pages,
                                 void* v_pages, int T, int H, int K, int dk, int dv, int page_size, hipStream_t stream);
 
@@ -323,4 +323,17 @@ int sa_delta_prepare(float* qkv, int T, int C, int G, int dk, const void* ab, in
 // S <- g S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.  Value head h reads q/k head h / (H / G).
 int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, const float* gates, int H, float* state,
                   int64_t state_stride, const int* seq_meta, int num_seqs, float* out, hipStream_t stream);
+
+// sa_paged_attention_decode and sa_paged_attention_prefill for softmax sums that hold one more term per query head,
+// exp(sinks[h]) (float32 [H]; null: none), without a value.
+int sa_paged_attention_decode_sink(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                                   const int* block_table, int table_stride, const int* seq_meta, int seq_begin,
+                                   int seq_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,
+                                   int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
+                                   void* workspace, int64_t workspace_bytes, const float* sinks, hipStream_t stream);
+int sa_paged_attention_prefill_sink(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                                    const int* block_table, int table_stride, const int* seq_meta, int unit_begin,
+                                    int unit_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,
+                                    int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
+                                    void* workspace, int64_t workspace_bytes, const float* sinks, hipStream_t stream);
 }

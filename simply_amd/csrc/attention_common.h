@@ -50,7 +50,8 @@ __device__ __forceinline__ float sum_over_row_lanes(float x) {
 // as many as it takes (num_ranges at most); a group with one range has written `out` itself and is skipped.
 int attention_merge_ranges(const float* workspace, int num_ranges, int hd, const SeqMeta* units, int unit_begin,
                            int unit_count, int max_q_len, bf16* out, int64_t out_stride, int Kh, int G,
-                           hipStream_t stream, int chunk_tiles = 0, int group = 1, int window = 0);
+                           hipStream_t stream, int chunk_tiles = 0, int group = 1, int window = 0,
+                           const float* sinks = nullptr);
 
 // The keys [lo, hi) that some row of the units [first, first + group) sees, and their request's slot.  False: no
 // rows.

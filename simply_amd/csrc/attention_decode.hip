@@ -43,7 +43,8 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ seq_meta, int seq_begin,
     bf16* __restrict__ out, int64_t out_stride, int Kh, int G, int page_size, int window, float soft_cap,
-    float* __restrict__ workspace) {
+    float* __restrict__ workspace, const float* __restrict__ sinks) {
+  // sinks (or null): one logit per query head that joins the softmax's sum and has no value
   constexpr int HD = NDC * 32;
   constexpr int NDB = HD / 16;  // output blocks of 16 dimensions
   __shared__ __align__(16) float o_s[2][16][HD + 4];   // a wave's output [row][d], while two waves are merged (rows of 16-byte pieces)
@@ -298,7 +299,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   if (wave == 0 && row_ok) {
     if (KS == 1) {
       bf16* op = out + static_cast<size_t>(sm.q_start + qi) * out_stride + static_cast<size_t>(kh * G + g) * HD;
-      const float inv = 1.f / l_run;
+      const float inv = 1.f / (sinks != nullptr ? l_run + __expf(sinks[kh * G + g] - m_run) : l_run);
 #pragma unroll
       for (int db = 0; db < NDB; ++db)
 #pragma unroll
@@ -322,7 +323,8 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
 __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float* __restrict__ workspace, int KS, int HD,
                                                                     const SeqMeta* __restrict__ seq_meta, int seq_begin,
                                                                     bf16* __restrict__ out, int64_t out_stride, int Kh,
-                                                                    int G, int chunk_tiles, int group, int window) {
+                                                                    int G, int chunk_tiles, int group, int window,
+                                                                    const float* __restrict__ sinks) {
   __shared__ float w_s[kMaxSplits];
   __shared__ float scratch[16];
   __shared__ float4 part_s[256];
@@ -395,7 +397,7 @@ __global__ __launch_bounds__(256) void paged_attention_merge_kernel(const float*
   }
   const int oq = orow / G, og = orow % G;
   bf16* op = out + static_cast<size_t>(sm.q_start + oq) * out_stride + static_cast<size_t>(kh * G + og) * HD;
-  const float inv = 1.f / Lg;
+  const float inv = 1.f / (sinks != nullptr ? Lg + __expf(sinks[kh * G + og] - Mg) : Lg);
   op[4 * c] = float_to_bf16(o.x * inv);
   op[4 * c + 1] = float_to_bf16(o.y * inv);
   op[4 * c + 2] = float_to_bf16(o.z * inv);
@@ -445,7 +447,7 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
                            const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                            float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
-                           hipStream_t stream) {
+                           hipStream_t stream, const float* sinks) {
   if (seq_count == 0) return 0;
   const int G = H / Kh;
   const int units = seq_count * Kh;
@@ -464,7 +466,7 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
 #define SA_LAUNCH(NDC)                                                                                              \
   paged_attention_decode_kernel<NDC><<<grid, 256, 0, stream>>>(qp, q_stride, kp, vp, block_table, table_stride, sm, \
                                                                seq_begin, op, out_stride, Kh, G, page_size, window,  \
-                                                               soft_cap, ws)
+                                                               soft_cap, ws, sinks)
   if (hd == 64) SA_LAUNCH(2);
   else if (hd == 128) SA_LAUNCH(4);
   else if (hd == 256) SA_LAUNCH(8);
@@ -474,7 +476,9 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
   }
 #undef SA_LAUNCH
   if (check_launch("paged_attention_decode")) return 1;
-  if (KS > 1) return attention_merge_ranges(ws, KS, hd, sm, seq_begin, seq_count, max_q_len, op, out_stride, Kh, G, stream);
+  if (KS > 1)
+    return attention_merge_ranges(ws, KS, hd, sm, seq_begin, seq_count, max_q_len, op, out_stride, Kh, G, stream, 0, 1, 0,
+                                  sinks);
   return 0;
 }
 
@@ -538,7 +542,8 @@ __global__ __launch_bounds__(256) void paged_attention_merge_rows_kernel(const f
                                                                          int HD, const SeqMeta* __restrict__ seq_meta,
                                                                          int seq_begin, bf16* __restrict__ out,
                                                                          int64_t out_stride, int Kh, int G,
-                                                                         int chunk_tiles, int group, int window) {
+                                                                         int chunk_tiles, int group, int window,
+                                                                         const float* __restrict__ sinks) {
   const int tid = threadIdx.x, kh = blockIdx.x, z = blockIdx.y;
   const SeqMeta sm = seq_meta[seq_begin + z];
   const int orow = tid / 16, part = tid % 16;
@@ -560,8 +565,8 @@ __global__ __launch_bounds__(256) void paged_attention_merge_rows_kernel(const f
     const float my = base[y * stride + HD];
     Lg += my == -INFINITY ? 0.f : base[y * stride + HD + 1] * __expf(my - Mg);
   }
-  const float inv = 1.f / Lg;
   const int oq = orow / G, og = orow % G;
+  const float inv = 1.f / (sinks != nullptr ? Lg + __expf(sinks[kh * G + og] - Mg) : Lg);
   bf16* op = out + static_cast<size_t>(sm.q_start + oq) * out_stride + static_cast<size_t>(kh * G + og) * HD;
   for (int d = part * 4; d < HD; d += 64) {
     float o[4] = {0.f, 0.f, 0.f, 0.f};
@@ -581,16 +586,16 @@ __global__ __launch_bounds__(256) void paged_attention_merge_rows_kernel(const f
 
 int attention_merge_ranges(const float* workspace, int num_ranges, int hd, const SeqMeta* units, int unit_begin,
                            int unit_count, int max_q_len, bf16* out, int64_t out_stride, int Kh, int G,
-                           hipStream_t stream, int chunk_tiles, int group, int window) {
+                           hipStream_t stream, int chunk_tiles, int group, int window, const float* sinks) {
   const int max_rows = G * max_q_len < 16 ? G * max_q_len : 16;
   if (max_rows > 4 && num_ranges <= 64) {
     paged_attention_merge_rows_kernel<<<dim3(Kh, unit_count), 256, 0, stream>>>(
-        workspace, num_ranges, hd, units, unit_begin, out, out_stride, Kh, G, chunk_tiles, group, window);
+        workspace, num_ranges, hd, units, unit_begin, out, out_stride, Kh, G, chunk_tiles, group, window, sinks);
     return check_launch("paged_attention_merge_rows");
   }
   // one workgroup per row: rows beyond the longest unit's are not launched
   paged_attention_merge_kernel<<<dim3(Kh, unit_count, max_rows), 256, 0, stream>>>(
-      workspace, num_ranges, hd, units, unit_begin, out, out_stride, Kh, G, chunk_tiles, group, window);
+      workspace, num_ranges, hd, units, unit_begin, out, out_stride, Kh, G, chunk_tiles, group, window, sinks);
   return check_launch("paged_attention_merge");
 }
 

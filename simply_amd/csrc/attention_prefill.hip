@@ -58,7 +58,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ units, int unit_begin,
     bf16* __restrict__ out, int64_t out_stride, int Kh, int G, int page_size, int window, float soft_cap,
-    float* __restrict__ workspace, int chunk_tiles) {
+    float* __restrict__ workspace, int chunk_tiles, const float* __restrict__ sinks) {
+  // sinks (or null): one logit per query head that joins the softmax's sum and has no value
   constexpr int HD = NDC * 32;
   constexpr int NDB = HD / 16;            // output blocks of 16 dimensions
   constexpr int CPW = NDC / 2;            // KiB chunks of keys (and of values) per wave and tile
@@ -376,6 +377,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
     if (!row_ok[j]) continue;
     if (num_chunks == 1) {
       bf16* op = out + static_cast<size_t>(q_row[j]) * out_stride + static_cast<size_t>(kh * G + g) * HD;
+      if (sinks != nullptr) l += __builtin_amdgcn_exp2f(sinks[kh * G + g] * kLog2e - m_run[j]);
       const float inv = 1.f / l;
 #pragma unroll
       for (int db = 0; db < NDB; ++db) {
@@ -418,7 +420,7 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
                             const int* block_table, int table_stride, const int* units, int unit_begin, int unit_count,
                             void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                             float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
-                            hipStream_t stream) {
+                            hipStream_t stream, const float* sinks) {
   constexpr int R = kPrefillRowTiles;
   constexpr int kGroup = prefill::kWaves * R;
   if (unit_count == 0) return 0;
@@ -464,11 +466,11 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
     if (soft_cap > 0.f)                                                                                             \
       prefill::paged_attention_prefill_kernel<NDC, R, true><<<grid, 256, 0, stream>>>(                              \
           qp, q_stride, kp, vp, block_table, table_stride, um, unit_begin, op, out_stride, Kh, G, page_size, window, \
-          soft_cap, ws, chunk);                                                                                     \
+          soft_cap, ws, chunk, sinks);                                                                              \
     else                                                                                                            \
       prefill::paged_attention_prefill_kernel<NDC, R, false><<<grid, 256, 0, stream>>>(                             \
           qp, q_stride, kp, vp, block_table, table_stride, um, unit_begin, op, out_stride, Kh, G, page_size, window, \
-          soft_cap, ws, chunk);                                                                                     \
+          soft_cap, ws, chunk, sinks);                                                                              \
   } while (0)
   if (hd == 64) SA_LAUNCH(2);
   else if (hd == 128) SA_LAUNCH(4);
@@ -481,7 +483,7 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
   if (check_launch("paged_attention_prefill")) return 1;
   if (KS > 1)
     return attention_merge_ranges(ws, KS, hd, um, unit_begin, unit_count, max_q_len, op, out_stride, Kh, G, stream, chunk,
-                                  kGroup, window);
+                                  kGroup, window, sinks);
   return 0;
 }
 

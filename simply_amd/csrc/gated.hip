@@ -84,14 +84,15 @@ __global__ void activation_kernel(void* __restrict__ x, int dtype, int64_t strid
 // ------------------------------------------------------------------ queries and keys: partial rotation, unit RMS
 // One wave per (token, head) of a fused projection row [H * dk queries | K * dk keys | K * dv values | ...].
 //   q, k: the first rot_dims dimensions are rotated in pairs (i, i + rot_dims / 2) by position * inv_freq[i], the
-//         others pass; then the head is divided by sqrt(mean(x^2) + eps) (eps < 0: left as it is).  Queries go back
-//         in place, keys into the key pages.
+//         others pass; then the head is divided by sqrt(mean(x^2) + eps) (eps < 0: left as it is).  Queries, times
+//         q_mult (the scores' factor, for attention kernels that have none), go back in place, keys into the key pages.
 //   v:    v <- (1 - lambda) v + lambda v_first (v_first null: v as it is), into the value pages (transposed).
 constexpr int kQkPerLane = 8;  // key sizes up to 512
 template <typename T>
 __global__ __launch_bounds__(kWave) void qk_norm_rope_cache_write_kernel(
     T* __restrict__ proj, int64_t row_stride, const int* __restrict__ positions, const float* __restrict__ inv_freq,
-    int rot_dims, float eps, const T* __restrict__ v_first, int64_t v_first_stride, const void* __restrict__ lambda,
+    int rot_dims, float eps, float q_mult, const T* __restrict__ v_first, int64_t v_first_stride,
+    const void* __restrict__ lambda,
     int lambda_dtype, const int64_t* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages,
     int H, int K, int dk, int dv, int page_size) {
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(kWave) void qk_norm_rope_cache_write_kernel(
 #pragma unroll
       for (int j = 0; j < kQkPerLane; ++j) {
         const int i = lane + j * kWave;
-        if (i < dk) src[i] = from_float<T>(o[j] * r);
+        if (i < dk) src[i] = from_float<T>(o[j] * r * q_mult);
       }
       return;
     }
@@ -210,8 +211,8 @@ extern "C" int sa_activation(void* x, int dtype, int64_t stride, int T, int N, i
 }
 
 extern "C" int sa_qk_norm_rope_cache_write(void* proj, int dtype, int64_t row_stride, const int* positions,
-                                           const float* inv_freq, int rot_dims, float eps, const void* v_first,
-                                           int64_t v_first_stride, const void* lambda, int lambda_dtype,
+                                           const float* inv_freq, int rot_dims, float eps, float q_mult,
+                                           const void* v_first, int64_t v_first_stride, const void* lambda, int lambda_dtype,
                                            const int64_t* slot_mapping, void* k_pages, void* v_pages, int T, int H,
                                            int K, int dk, int dv, int page_size, hipStream_t stream) {
   if (T == 0) return 0;
@@ -230,12 +231,12 @@ extern "C" int sa_qk_norm_rope_cache_write(void* proj, int dtype, int64_t row_st
   const dim3 grid(T, H + 2 * K);
   if (dtype == kF32)
     qk_norm_rope_cache_write_kernel<float><<<grid, kWave, 0, stream>>>(
-        static_cast<float*>(proj), row_stride, positions, inv_freq, rot_dims, eps, static_cast<const float*>(v_first),
+        static_cast<float*>(proj), row_stride, positions, inv_freq, rot_dims, eps, q_mult, static_cast<const float*>(v_first),
         v_first_stride, lambda, lambda_dtype, slot_mapping, static_cast<float*>(k_pages), static_cast<float*>(v_pages),
         H, K, dk, dv, page_size);
   else if (dtype == kBF16)
     qk_norm_rope_cache_write_kernel<bf16><<<grid, kWave, 0, stream>>>(
-        static_cast<bf16*>(proj), row_stride, positions, inv_freq, rot_dims, eps, static_cast<const bf16*>(v_first),
+        static_cast<bf16*>(proj), row_stride, positions, inv_freq, rot_dims, eps, q_mult, static_cast<const bf16*>(v_first),
         v_first_stride, lambda, lambda_dtype, slot_mapping, static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), H,
         K, dk, dv, page_size);
   else

@@ -59,7 +59,11 @@ _SIGNATURES = {
     "sa_residual_add_norm": [_P, _I, _L, _P, _I, _F, _I, _F, _P, _P, _I, _I, _I, _P],
     "sa_gated_heads": [_P, _I, _L, _P, _I, _L, _P, _I, _F, _I, _P, _I, _L, _I, _I, _I, _P],
     "sa_activation": [_P, _I, _L, _I, _I, _I, _P],
-    "sa_qk_norm_rope_cache_write": [_P, _I, _L, _P, _P, _I, _F, _P, _L, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "sa_qk_norm_rope_cache_write": [_P, _I, _L, _P, _P, _I, _F, _F, _P, _L, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+    "sa_paged_attention_decode_sink": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P,
+                                       _L, _P, _P],
+    "sa_paged_attention_prefill_sink": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P,
+                                        _L, _P, _P],
     "sa_short_conv_silu": [_P, _I, _L, _P, _I, _I, _P, _L, _P, _I, _I, _P, _I, _I, _P],
     "sa_delta_prepare": [_P, _I, _I, _I, _I, _P, _I, _L, _P, _P, _I, _I, _P, _P],
     "sa_delta_rule": [_P, _I, _I, _I, _I, _P, _I, _P, _L, _P, _I, _P, _P],

@@ -620,8 +620,8 @@ def decode_attention_takes(q: torch.Tensor, k_pages: torch.Tensor, num_heads: in
 
 
 def _attention_units(entry: str, q, k_pages, v_pages, block_table, seq_meta, begin, count, num_heads, window, soft_cap,
-                     max_kv_len, max_q_len, out, num_splits):
-    _dev(q, k_pages, v_pages, block_table, seq_meta, out)
+                     max_kv_len, max_q_len, out, num_splits, sinks=None):
+    _dev(q, k_pages, v_pages, block_table, seq_meta, out, sinks)
     name = entry[3:]
     if q.dtype != torch.bfloat16:
         raise KernelError(f"{name}: bfloat16 only")
@@ -637,6 +637,15 @@ def _attention_units(entry: str, q, k_pages, v_pages, block_table, seq_meta, beg
         raise KernelError(f"{name}: bad output")
     out_stride = _rows(out, f"{name}: out")
     ws = _workspace(q.device)
+    if sinks is not None:
+        # one more term exp(sinks[h]) in every softmax sum of query head h, without a value
+        if sinks.dtype != torch.float32 or sinks.numel() != num_heads or not sinks.is_contiguous():
+            raise KernelError(f"{name}: sinks must be contiguous float32, one per query head")
+        _lib.call(entry + "_sink", _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+                  block_table.stride(0), _ptr(seq_meta), begin, count, _ptr(out), out_stride, num_heads, Kh, hd,
+                  page_size, int(window or 0), float(soft_cap or 0.0), int(max_kv_len), int(max_q_len), int(num_splits),
+                  _ptr(ws), ws.numel(), _ptr(sinks), _stream())
+        return out
     _lib.call(entry, _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
               block_table.stride(0), _ptr(seq_meta), begin, count, _ptr(out), out_stride, num_heads, Kh, hd,
               page_size, int(window or 0), float(soft_cap or 0.0), int(max_kv_len), int(max_q_len), int(num_splits),
@@ -647,11 +656,12 @@ def _attention_units(entry: str, q, k_pages, v_pages, block_table, seq_meta, beg
 def paged_attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                            seq_meta: torch.Tensor, seq_begin: int, seq_count: int, num_heads: int, *,
                            window: int | None, soft_cap: float | None, max_kv_len: int, max_q_len: int,
-                           out: torch.Tensor, num_splits: int = 0) -> torch.Tensor:
+                           out: torch.Tensor, num_splits: int = 0, sinks: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of requests seq_begin .. seq_begin + seq_count - 1 of seq_meta, each with few tokens
-    ((heads per key head) * tokens <= 16).  q and out are the whole step's rows."""
+    ((heads per key head) * tokens <= 16).  q and out are the whole step's rows.  sinks: float32 [H], one more term
+    exp(sinks[h]) in every softmax sum, without a value."""
     return _attention_units("sa_paged_attention_decode", q, k_pages, v_pages, block_table, seq_meta, seq_begin,
-                            seq_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits)
+                            seq_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits, sinks)
 
 
 def prefill_units_per_group() -> int:
@@ -662,7 +672,7 @@ def prefill_units_per_group() -> int:
 def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                             units: torch.Tensor, unit_begin: int, unit_count: int, num_heads: int, *,
                             window: int | None, soft_cap: float | None, max_kv_len: int, max_q_len: int,
-                            out: torch.Tensor, num_splits: int = 0) -> torch.Tensor:
+                            out: torch.Tensor, num_splits: int = 0, sinks: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of portions of prompts cut into units of few tokens ((heads per key head) * tokens <= 16), rows
     unit_begin .. unit_begin + unit_count - 1 of `units` in the layout of seq_meta.  One workgroup takes a group of
     consecutive units, which must belong to one request (units without tokens fill up the last group), and
@@ -670,7 +680,7 @@ def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     if unit_count % prefill_units_per_group():
         raise KernelError(f"paged_attention_prefill: units come in groups of {prefill_units_per_group()}")
     return _attention_units("sa_paged_attention_prefill", q, k_pages, v_pages, block_table, units, unit_begin,
-                            unit_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits)
+                            unit_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits, sinks)
 
 
 def paged_attention_sink(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
@@ -786,11 +796,12 @@ def qk_norm_rope_cache_write(proj: torch.Tensor, positions: torch.Tensor, inv_fr
                              eps: float | None, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, *,
                              v_first: torch.Tensor | None = None, v_mix: torch.Tensor | None = None,
                              slot_mapping: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
-                             v_pages: torch.Tensor | None = None) -> torch.Tensor:
+                             v_pages: torch.Tensor | None = None, q_mult: float = 1.0) -> torch.Tensor:
     """In place on fused projection rows [H * dk | K * dk | K * dv | ...]: queries and keys rotated on their first
     rot_dims dimensions (angle position * inv_freq[i] for the pair (i, i + rot_dims / 2)), then divided by their root
     mean square (eps None: not); values mixed, (1 - v_mix) v + v_mix v_first (v_first [T, K * dv] rows of another
-    layer, v_mix a tensor of one element), keys and values written into the pages."""
+    layer, v_mix a tensor of one element), keys and values written into the pages.  q_mult: a factor on the
+    queries (the scores' factor, for an attention kernel that has none of its own)."""
     _dev(proj, positions, inv_freq, v_first, v_mix, slot_mapping, k_pages, v_pages)
     stride = _rows(proj, "qk_norm_rope_cache_write: proj")
     T = proj.shape[0]
@@ -822,7 +833,7 @@ def qk_norm_rope_cache_write(proj: torch.Tensor, positions: torch.Tensor, inv_fr
                               "[T, K * dv] of the projection's type")
         vfs = _rows(v_first, "qk_norm_rope_cache_write: v_first")
     _lib.call("sa_qk_norm_rope_cache_write", _ptr(proj), _code(proj), stride, _ptr(positions), _ptr(inv_freq),
-              int(rot_dims), float(eps) if eps is not None else -1.0, _ptr(v_first), vfs, _ptr(v_mix),
+              int(rot_dims), float(eps) if eps is not None else -1.0, float(q_mult), _ptr(v_first), vfs, _ptr(v_mix),
               _code(v_mix) if v_mix is not None else 0, _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), T, H, K, dk,
               dv, int(page_size), _stream())
     return proj

@@ -152,6 +152,7 @@ class SinkAttention(Mixer):
         self.in_proj = as_product_weight(torch.cat(rows, dim=0).contiguous())
         self.o_proj = as_product_weight(tensors["o_proj"])
         self.sink = tensors["sink"].contiguous() if self.sinks else None
+        self.sink_f32 = self.sink.to(torch.float32) if self.sinks else None   # what the MFMA kernels read
         self.vmix = tensors["vmix"].reshape(1).contiguous() if self.value_mix is not None else None
         if self.position_encoding is not None:
             self.position_encoding.to_device(tensors["o_proj"].device)
@@ -171,14 +172,29 @@ class SinkAttention(Mixer):
             if v_first is None:
                 raise RuntimeError(f"sink_attention: no earlier layer of the step has left {self.value_mix_key!r}")
         write = cache.write
+        # the bfloat16 MFMA kernels take values of the keys' size (64, 128 or 256) in pages of a multiple of 16 keys;
+        # they have no factor on the scores, so the queries carry it
+        mfma = dk == dv and proj.dtype == torch.bfloat16 and ops.decode_attention_takes(proj, cache.k_pages, H, 1)
         ops.qk_norm_rope_cache_write(proj, ctx.positions, inv_freq, rot_dims, self.qk_norm_eps, H, K, dk, dv,
                                      v_first=v_first, v_mix=self.vmix if v_first is not None else None,
                                      slot_mapping=group.slot_mapping if write else None,
-                                     k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
+                                     k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None,
+                                     q_mult=self.scale if mfma else 1.0)
         if self.value_mix == "source":
             ctx.carry[self.value_mix_key] = proj[:, v_at:v_at + K * dv]
-        o = ops.paged_attention_sink(proj, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq, ctx.positions,
-                                     H, scale=self.scale, sinks=self.sink, window=self.window)
+        if mfma:
+            o = torch.empty((proj.shape[0], H * dv), dtype=proj.dtype, device=proj.device)
+            units, few, many, max_q = ctx.attention_units(16 // (H // K), ops.prefill_units_per_group())
+            kw = dict(window=self.window, soft_cap=None, max_kv_len=ctx.max_kv_len, max_q_len=max_q, out=o,
+                      sinks=self.sink_f32)
+            if few:
+                ops.paged_attention_decode(proj, cache.k_pages, cache.v_pages, group.block_table, units, 0, few, H, **kw)
+            if many:
+                ops.paged_attention_prefill(proj, cache.k_pages, cache.v_pages, group.block_table, units, few, many, H,
+                                            **kw)
+        else:
+            o = ops.paged_attention_sink(proj, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq,
+                                         ctx.positions, H, scale=self.scale, sinks=self.sink, window=self.window)
         if self.output_gate:
             g_at = v_at + K * dv
             ops.gated_heads(o, proj[:, g_at:g_at + H * dv], H, dv, kind=ops.GATE_SIGMOID, out=o)

@@ -42,6 +42,13 @@ def test_attention_part(dtype):
     mech.attention_part(DEV, dtype)
 
 
+def test_attention_part_on_the_matrix_cores():
+    """Values of the keys' size (64) in pages of 16 keys, bfloat16: the MFMA kernels run, few rows a request and
+    portions of prompts, with their key ranges merged, the sinks in every sum and the scores' factor in the queries."""
+    mech.attention_part(DEV, torch.bfloat16, sizes=(96, 8, 2, 64, 64), length=700,
+                        cuts=([700], [300, 1, 1, 1, 2, 395], [640] + [1] * 60, [17] * 41 + [3]))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_delta_part(dtype):
     mech.delta_part(DEV, dtype)
@@ -57,6 +64,14 @@ def test_cuts_match_plain(tmp_path, name, dtype):
 @pytest.mark.parametrize("name", ["mixed", "only_delta", "aligned"])
 def test_batches_match_alone(tmp_path, name, dtype):
     cases.batches_match_alone(tmp_path, DEV, name, dtype)
+
+
+def test_pages_of_sixteen_keys(tmp_path):
+    """The sizes that the bfloat16 MFMA attention kernels take, in pages of 16 keys: cuts of a prompt, unequal
+    requests in a tight pool, long decoding."""
+    cases.cuts_match_plain(tmp_path, DEV, "aligned", "bfloat16", length=70, page_size=16)
+    cases.batches_match_alone(tmp_path / "b", DEV, "aligned", "bfloat16", page_size=16)
+    cases.long_decoding(tmp_path / "l", DEV, "aligned", "bfloat16", steps=150, page_size=16)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

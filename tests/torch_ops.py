@@ -272,7 +272,7 @@ def activation_(x, activation):
 
 
 def qk_norm_rope_cache_write(proj, positions, inv_freq, rot_dims, eps, num_heads, num_kv_heads, key_dim, value_dim, *,
-                             v_first=None, v_mix=None, slot_mapping=None, k_pages=None, v_pages=None):
+                             v_first=None, v_mix=None, slot_mapping=None, k_pages=None, v_pages=None, q_mult=1.0):
     T = proj.shape[0]
     H, K, dk, dv = num_heads, num_kv_heads, key_dim, value_dim
     qk = _f(proj[:, :(H + K) * dk]).reshape(T, H + K, dk).clone()
@@ -285,7 +285,7 @@ def qk_norm_rope_cache_write(proj, positions, inv_freq, rot_dims, eps, num_heads
         qk[..., half:rot_dims] = b * c + a * s
     if eps is not None:
         qk = qk / torch.sqrt((qk * qk).mean(-1, keepdim=True) + eps)
-    proj[:, :H * dk] = qk[:, :H].reshape(T, H * dk).to(proj.dtype)
+    proj[:, :H * dk] = (qk[:, :H] * q_mult).reshape(T, H * dk).to(proj.dtype)
     if k_pages is None:
         return proj
     P = k_pages.shape[2]

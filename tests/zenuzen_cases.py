@@ -139,19 +139,19 @@ def plain_weights(model_dir, dtype):
 # --------------------------------------------------------------------------- bodies
 
 
-def cuts_match_plain(tmp_path, device, name, dtype="float32", length=45):
+def cuts_match_plain(tmp_path, device, name, dtype="float32", length=45, page_size=4):
     d = write_model(name, str(tmp_path / name))
     w, cfg = plain_weights(d, dtype)
     tokens = random_tokens(length, cfg["vocab"], 7)
     want = plain.forward(w, cfg, tokens)
-    ex = make_executor(d, device, dtype)
+    ex = make_executor(d, device, dtype, page_size=page_size)
     n = length
     for cuts in ([n], [n - 32] + [1] * 32, [7, 5, 3, 2, 11, 2, 2, n - 32], [2] * (n // 2) + [1] * (n % 2), [1] * n):
         got = run_cut(ex, "r", tokens, cuts)
         assert_close_logits(got, want, dtype, (name, cuts))
 
 
-def batches_match_alone(tmp_path, device, name, dtype="float32"):
+def batches_match_alone(tmp_path, device, name, dtype="float32", page_size=4):
     """Requests of unequal length run together, portions beside single tokens, in a pool so tight that pages and
     state slots are given back and used again (freed pages are filled with NaN): each request's logits are those of
     the request alone."""
@@ -162,7 +162,8 @@ def batches_match_alone(tmp_path, device, name, dtype="float32"):
     toks = {r: random_tokens(n, V, 100 + i) for i, (r, n) in enumerate(lengths.items())}
     want = {r: plain.forward(w, cfg, t) for r, t in toks.items()}
     # at most three live at a time: 3 slots, and pages for 37 + 30 + 22 tokens rounded up
-    ex = make_executor(d, device, dtype, page_size=4, num_pages=26, batch=3, max_len=40, poison=True)
+    ex = make_executor(d, device, dtype, page_size=page_size, num_pages=26 if page_size == 4 else 8, batch=3, max_len=48,
+                       poison=True)
     schedule = [
         [("a", 11), ("b", 3), ("c", 1)],          # c ends: its slot goes to d
         [("a", 2), ("b", 1), ("d", 5)],

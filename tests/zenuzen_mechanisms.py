@@ -218,22 +218,27 @@ def _load(part, dtype, device, seed, scale=0.3, fixed=None):
     return {k: v.double().cpu() for k, v in tensors.items()}
 
 
-def attention_part(device, dtype):
-    """The attention mixer with a cache of its own, whole and in portions that cut pages, against the plain mixer."""
-    D, H, K, dk, dv, eps = 40, 4, 2, 12, 20, 1e-5
+def attention_part(device, dtype, sizes=(40, 4, 2, 12, 20), length=50, cuts=([50], [15, 1, 1, 2, 31], [2] * 25)):
+    """The attention mixer with a cache of its own, whole and in portions that cut pages, against the plain mixer.
+    The sinks are large, so that one that is left out shows."""
+    D, H, K, dk, dv = sizes
+    eps = 1e-5
     params = dict(hidden_size=D, num_heads=H, num_kv_heads=K, key_dim=dk, value_dim=dv, scale=0.5, sinks=True,
                   qk_norm_eps=eps, output_gate=True, value_mix=None,
                   position_encoding=PartSpec("partial_rope", {"head_dim": dk, "dims": 6, "base": 50.0}))
     part = registry.MIXERS.build("sink_attention", **params)
-    t = _load(part, dtype, device, 30)
+    t = _load(part, dtype, device, 30, fixed={"sink": torch.linspace(-2.0, 4.0, H, dtype=torch.float64)})
     w = {"p.q": t["q_proj"], "p.k": t["k_proj"], "p.v": t["v_proj"], "p.g": t["gate_proj"], "p.o": t["o_proj"],
          "p.sink": t["sink"]}
     mc = {"heads": H, "kv_heads": K, "dim": dk, "vdim": dv, "scale": 0.5, "rot": {"dims": 6, "base": 50.0}}
-    x = rand((50, D), 31).to(dtype)
-    want = plain.attention_mixer(x.double(), torch.arange(50), w, "p.", mc, eps, {})
+    x = rand((length, D), 31).to(dtype)
+    want = plain.attention_mixer(x.double(), torch.arange(length), w, "p.", mc, eps, {})
+    without = plain.attention_mixer(x.double(), torch.arange(length), dict(w, **{"p.sink": w["p.sink"] - 30.0}), "p.", mc,
+                                    eps, {})
+    assert float((without - want).abs().max() / want.abs().max()) > 0.3     # the sinks matter
     tol = 3e-5 if dtype == torch.float32 else 4e-2
-    for cuts in ([50], [15, 1, 1, 2, 31], [2] * 25):
-        close(run_mixer(part, x.to(device), cuts, dtype, device), want, tol, str(cuts))
+    for c in cuts:
+        close(run_mixer(part, x.to(device), c, dtype, device), want, tol, str(c))
 
 
 def delta_part(device, dtype):
