@@ -109,16 +109,27 @@ __global__ __launch_bounds__(kWave) void delta_prepare_kernel(float* __restrict_
 // Columns are independent of each other; a column's sums run within a lane over its rows in increasing order, in
 // four partial sums that are added in a fixed order, then across the lanes by data-parallel primitives in a fixed
 // order: nothing depends on how the tokens are cut into steps or on the batch.  The chain of dependent operations
-// per token is what bounds a prompt's time (tokens follow one another): 16 lanes per column keep it short where a
+// per token, and the instructions that one wave issues for it, are what bound a prompt's time (tokens follow one
+// another, and a head's columns are all the waves there are): 16 or 32 lanes per column keep both short where a
 // column has 64 rows or more.
 constexpr int kRuleTokens = 16;
 template <int LPC>
 __device__ __forceinline__ float lanes_sum(float v) {
   v += lane_exchange<0xB1>(v);   // quad_perm [1, 0, 3, 2]
   v += lane_exchange<0x4E>(v);   // quad_perm [2, 3, 0, 1]
-  if (LPC == 16) {
+  if (LPC >= 16) {
     v += lane_exchange<0x141>(v);  // row_half_mirror
     v += lane_exchange<0x140>(v);  // row_mirror
+  }
+  if (LPC >= 32) {   // two rows of 16 lanes: gfx950's row swap brings the neighbouring row's sum
+    const unsigned u = __float_as_uint(v);
+    const auto rows = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    v = __uint_as_float(rows[0]) + __uint_as_float(rows[1]);
+  }
+  if (LPC == 64) {   // and the other half of the wave
+    const unsigned u = __float_as_uint(v);
+    const auto halves = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    v = __uint_as_float(halves[0]) + __uint_as_float(halves[1]);
   }
   return v;
 }
@@ -146,52 +157,93 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
     s[r] = (live && i < dk) ? S[static_cast<size_t>(i) * dv + col] : 0.f;
   }
   const int v_at = 2 * G * dk + h * dv;
+  // A tile's q, k, v and gates are asked for a tile ahead, into registers, and put into LDS when the tile's turn
+  // comes: the loads are under way while the tile before is worked through.
+  constexpr int PQ = kRuleTokens * DK / 256, PV = (kRuleTokens * COLS + 255) / 256;
+  float pq[PQ], pk[PQ], pv[PV], pg = 0.f;
+  auto fetch = [&](int t0) __attribute__((always_inline)) {
+    const int tn = count - t0 < kRuleTokens ? count - t0 : kRuleTokens;
+#pragma unroll
+    for (int i = 0; i < PQ; ++i) {
+      const int idx = tid + i * 256, j = idx / DK, d = idx % DK;
+      const bool ok = j < tn && d < dk;
+      const float* row = qkv + static_cast<size_t>(first + t0 + (ok ? j : 0)) * C;
+      pq[i] = ok ? row[qk_head * dk + d] : 0.f;
+      pk[i] = ok ? row[(G + qk_head) * dk + d] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < PV; ++i) {
+      const int idx = tid + i * 256, j = idx / COLS, c = blockIdx.z * COLS + idx % COLS;
+      const bool ok = idx < kRuleTokens * COLS && j < tn && c < dv;
+      pv[i] = ok ? qkv[static_cast<size_t>(first + t0 + j) * C + v_at + c] : 0.f;
+    }
+    pg = tid < 2 * tn ? gates[static_cast<size_t>(first + t0 + tid / 2) * 2 * H + (tid % 2) * H + h] : 0.f;
+  };
+  if (count > 0) fetch(0);
   for (int t0 = 0; t0 < count; t0 += kRuleTokens) {
     const int tn = count - t0 < kRuleTokens ? count - t0 : kRuleTokens;
     __syncthreads();
-    for (int idx = tid; idx < tn * DK; idx += 256) {
-      const int j = idx / DK, i = idx % DK;
-      const float* row = qkv + static_cast<size_t>(first + t0 + j) * C;
-      qs[j][i] = i < dk ? row[qk_head * dk + i] : 0.f;
-      ks[j][i] = i < dk ? row[(G + qk_head) * dk + i] : 0.f;
+#pragma unroll
+    for (int i = 0; i < PQ; ++i) {
+      const int idx = tid + i * 256;
+      qs[idx / DK][idx % DK] = pq[i];
+      ks[idx / DK][idx % DK] = pk[i];
     }
-    for (int idx = tid; idx < tn * COLS; idx += 256) {
-      const int j = idx / COLS, c = blockIdx.z * COLS + idx % COLS;
-      vs[j][idx % COLS] = c < dv ? qkv[static_cast<size_t>(first + t0 + j) * C + v_at + c] : 0.f;
+#pragma unroll
+    for (int i = 0; i < PV; ++i) {
+      const int idx = tid + i * 256;
+      if (idx < kRuleTokens * COLS) vs[idx / COLS][idx % COLS] = pv[i];
     }
-    if (tid < 2 * tn) bg[tid / 2][tid % 2] = gates[static_cast<size_t>(first + t0 + tid / 2) * 2 * H + (tid % 2) * H + h];
+    if (tid < 2 * kRuleTokens) bg[tid / 2][tid % 2] = pg;
     __syncthreads();
-    for (int j = 0; j < tn; ++j) {
-      const size_t t = static_cast<size_t>(first + t0 + j);
-      const float beta = bg[j][0], g = bg[j][1];
-      const float v = vs[j][tid / LPC];
-      float kr[R], qr[R];
+    if (t0 + kRuleTokens < count) fetch(t0 + kRuleTokens);
+    // the token's operands are read from LDS a token ahead, into one of two sets of registers in turn
+    struct Operands {
+      float k[R], q[R], v, beta, g;
+    };
+    auto read = [&](Operands& x, int j) __attribute__((always_inline)) {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        kr[r] = ks[j][r * LPC + part];
-        qr[r] = qs[j][r * LPC + part];
+        x.k[r] = ks[j][r * LPC + part];
+        x.q[r] = qs[j][r * LPC + part];
       }
+      x.v = vs[j][tid / LPC];
+      x.beta = bg[j][0];
+      x.g = bg[j][1];
+    };
+    auto token = [&](const Operands& x, int j) __attribute__((always_inline)) {
       float d[NACC];
 #pragma unroll
       for (int a = 0; a < NACC; ++a) d[a] = 0.f;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        s[r] *= g;
-        d[r % NACC] = fmaf(s[r], kr[r], d[r % NACC]);
+        s[r] *= x.g;
+        d[r % NACC] = fmaf(s[r], x.k[r], d[r % NACC]);
       }
       float dot = NACC == 4 ? (d[0] + d[1]) + (d[2] + d[3]) : d[0];
       dot = lanes_sum<LPC>(dot);
-      const float u = beta * (v - dot);
+      const float u = x.beta * (x.v - dot);
 #pragma unroll
       for (int a = 0; a < NACC; ++a) d[a] = 0.f;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        s[r] = fmaf(kr[r], u, s[r]);
-        d[r % NACC] = fmaf(s[r], qr[r], d[r % NACC]);
+        s[r] = fmaf(x.k[r], u, s[r]);
+        d[r % NACC] = fmaf(s[r], x.q[r], d[r % NACC]);
       }
       float o = NACC == 4 ? (d[0] + d[1]) + (d[2] + d[3]) : d[0];
       o = lanes_sum<LPC>(o);
-      if (live && part == 0) out[t * (static_cast<size_t>(H) * dv) + static_cast<size_t>(h) * dv + col] = o;
+      if (live && part == 0)
+        out[static_cast<size_t>(first + t0 + j) * (static_cast<size_t>(H) * dv) + static_cast<size_t>(h) * dv + col] = o;
+    };
+    Operands A, B;
+    read(A, 0);
+    for (int j = 0; j < tn; j += 2) {
+      if (j + 1 < tn) read(B, j + 1);
+      token(A, j);
+      if (j + 1 < tn) {
+        if (j + 2 < tn) read(A, j + 2);
+        token(B, j + 1);
+      }
     }
   }
 #pragma unroll
@@ -255,8 +307,8 @@ extern "C" int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, con
   if (dk <= 16) SA_DELTA_RULE(16, 4);
   else if (dk <= 32) SA_DELTA_RULE(32, 4);
   else if (dk <= 64) SA_DELTA_RULE(64, 16);
-  else if (dk <= 128) SA_DELTA_RULE(128, 16);
-  else SA_DELTA_RULE(256, 16);
+  else if (dk <= 128) SA_DELTA_RULE(128, 64);
+  else SA_DELTA_RULE(256, 64);
 #undef SA_DELTA_RULE
   return check_launch("delta_rule");
 }
