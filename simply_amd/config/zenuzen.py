@@ -120,8 +120,8 @@ class ZenuzenConfig:
     residual_mult: float
     norm_eps: float
     layers: tuple[ZenuzenLayer, ...]
-    #: not part of the design: what the engine may assume when nothing else limits a sequence
-    max_position: int = 1 << 20
+    #: not part of the design: the longest sequence that the engine plans for when --max_seq_len does not say
+    max_position: int = 8192
     eos_token_ids: tuple[int, ...] = ()
     initializer_range: float = 0.02
 
@@ -138,7 +138,7 @@ class ZenuzenConfig:
                   residual_mult=_get(d, "residual_mult", "top level", float),
                   norm_eps=_get(_get(d, "norm", "top level"), "eps", "norm", float),
                   layers=tuple(ZenuzenLayer.from_dict(l, i) for i, l in enumerate(layers)),
-                  max_position=int(d.get("max_position", 1 << 20)), eos_token_ids=eos_ids,
+                  max_position=int(d.get("max_position", 8192)), eos_token_ids=eos_ids,
                   initializer_range=float(d.get("initializer_range", 0.02)))
         cfg.validate()
         return cfg
@@ -160,7 +160,7 @@ class ZenuzenConfig:
                              "layers": [l.to_dict() for l in self.layers]}
         if self.eos_token_ids:
             d["eos_token_id"] = list(self.eos_token_ids)
-        if self.max_position != 1 << 20:
+        if self.max_position != 8192:
             d["max_position"] = self.max_position
         if self.initializer_range != 0.02:
             d["initializer_range"] = self.initializer_range

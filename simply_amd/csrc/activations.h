@@ -10,7 +10,8 @@ namespace sa {
 
 enum Activation : int { kActGeluTanh = 0, kActSilu = 1, kActSquaredRelu = 2, kNumActivations = 3 };
 
-constexpr int kEpilogueNone = 0, kEpilogueGated = 1, kEpilogueSoftCap = 2;
+// kEpilogueActivated: C = act(A.W^T), the product rounded to the output type first (a feed-forward without a gate)
+constexpr int kEpilogueNone = 0, kEpilogueGated = 1, kEpilogueSoftCap = 2, kEpilogueActivated = 3;
 // The epilogue argument of an entry point: its kind in the low four bits, the gated kind's activation above them.
 __host__ __device__ inline int epilogue_kind(int epilogue) { return epilogue & 15; }
 __host__ __device__ inline int epilogue_activation(int epilogue) { return epilogue >> 4; }

@@ -84,7 +84,8 @@ int sa_decode_slots(int B, const int* positions, const int* token_seq, const int
 
 // C[M, N] = epilogue(A[M, K] . W[N, K]^T).  epilogue 0: none; 1 + 16 * a: act(A.W^T) * (A.W2^T) with the activation
 // a of activations.h (0: tanh-approximated gelu, 1: silu, 2: squared relu), both products rounded to the output
-// type first; 2: cap * tanh(. / cap).  algo 0: the library chooses; 1: the generic 32-bit-ALU kernel; 2: the
+// type first; 2: cap * tanh(. / cap); 3 + 16 * a: act(A.W^T), the product rounded to the output type first (in
+// the wide kernel's epilogue where that kernel runs without a cut of K, else by a kernel behind the product).  algo 0: the library chooses; 1: the generic 32-bit-ALU kernel; 2: the
 // few-rows bfloat16 kernel; 3: the tiled bfloat16 MFMA kernel; 4: the wide-tile bfloat16 MFMA kernel for very
 // many rows (2, 3 and 4 refuse what they do not take).
 // packed: W (and W2) are tiled instead of row-major: [ceil(N / 16)][ceil(K / 32)][64][8] bfloat16, block (i, j)
@@ -228,6 +229,8 @@ namespace sa {
 int gemm_generic(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,
                  int c_dtype, int64_t ldc, int M, int N, int K, int epi, int act, float cap, int packed,
                  hipStream_t stream);
+// x = act(x) in place, row by row (the separate kernel behind products whose kernels have no such epilogue)
+int apply_activation(void* x, int dtype, int64_t stride, int M, int N, int act, hipStream_t stream);
 bool gemm_skinny_takes(int M, int N, int K, int64_t lda, const void* A, const void* W, const void* W2);
 // Expected microseconds of each bfloat16 product kernel for these sizes (epi: 0 none, 1 gated, 2 soft-cap); negative:
 // the kernel is not made for them.  The dispatcher runs the kernel with the smallest figure among those that take

@@ -196,6 +196,12 @@ extern "C" int sa_gated_heads(const void* x, int x_dtype, int64_t x_stride, cons
   return check_launch("gated_heads");
 }
 
+namespace sa {
+int apply_activation(void* x, int dtype, int64_t stride, int M, int N, int act, hipStream_t stream) {
+  return sa_activation(x, dtype, stride, M, N, act, stream);
+}
+}  // namespace sa
+
 extern "C" int sa_activation(void* x, int dtype, int64_t stride, int T, int N, int act, hipStream_t stream) {
   if (T == 0 || N == 0) return 0;
   SA_REQUIRE(T > 0 && N > 0 && stride >= N && T <= 65535 * 1024, "activation: bad sizes T=%d N=%d", T, N);

@@ -287,6 +287,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_wide_kernel(const bf16* __res
                  to_float(float_to_bf16(acc[i][2 * j + 1][v]));
         else
           x[v] = acc[i][j][v];
+        // (without another epilogue, act > 0 asks for the activation act - 1 of the product rounded to bfloat16)
+        if (EPI == 0 && act > 0) x[v] = gated_activation(act - 1, to_float(float_to_bf16(x[v])));
       }
       uint2 packed;
       packed.x = static_cast<uint32_t>(float_to_bf16(x[0]).bits) | (static_cast<uint32_t>(float_to_bf16(x[1]).bits) << 16);
@@ -440,7 +442,10 @@ int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, i
     *planes_left = ks;
     return 0;
   }
-  if (ks > 1) return gemm_sum_partials(ws, ks, C, kBF16, ldc, M, N, N, 0, 0, 0.f, stream);
+  if (ks > 1) {
+    if (gemm_sum_partials(ws, ks, C, kBF16, ldc, M, N, N, 0, 0, 0.f, stream)) return 1;
+    if (epi == 0 && act > 0) return apply_activation(C, kBF16, ldc, M, N, act - 1, stream);   // (the kernels with K cut have no such epilogue)
+  }
   return 0;
 }
 

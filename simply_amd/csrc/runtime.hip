@@ -41,10 +41,19 @@ static int gemm_routed(const void* A, int a_dtype, int64_t lda, const void* W, c
   SA_REQUIRE(M > 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
   SA_REQUIRE(lda >= K && ldc >= N, "gemm: leading dimensions lda=%lld ldc=%lld are below K=%d, N=%d", (long long)lda,
              (long long)ldc, K, N);
-  const int act = epilogue_activation(epilogue);
+  int act = epilogue_activation(epilogue);
   epilogue = epilogue_kind(epilogue);
-  SA_REQUIRE(epilogue >= 0 && epilogue <= 2, "gemm: unknown epilogue %d", epilogue);
-  SA_REQUIRE(act >= 0 && act < kNumActivations && (epilogue == 1 || act == 0), "gemm: unknown activation %d", act);
+  SA_REQUIRE(epilogue >= 0 && epilogue <= 3, "gemm: unknown epilogue %d", epilogue);
+  SA_REQUIRE(act >= 0 && act < kNumActivations && (epilogue == 1 || epilogue == 3 || act == 0),
+             "gemm: unknown activation %d", act);
+  // an activation without a gate: the product as without an epilogue, the activation in the wide kernel's epilogue
+  // or, behind every other kernel, by a kernel of its own
+  const int activated = epilogue == kEpilogueActivated ? act + 1 : 0;
+  if (activated) {
+    SA_REQUIRE(planes_left == nullptr && W2 == nullptr, "gemm: an activated product is summed here and has one weight");
+    epilogue = kEpilogueNone;
+    act = 0;
+  }
   SA_REQUIRE(epilogue != 1 || (W2 != nullptr) != (packed != 0),
              "gemm: the gated epilogue takes two row-major weights, or one tiled weight that holds both");
   SA_REQUIRE(epilogue != 2 || cap > 0.f, "gemm: the soft-cap epilogue needs a positive cap");
@@ -81,15 +90,19 @@ static int gemm_routed(const void* A, int a_dtype, int64_t lda, const void* W, c
         kernel = 2 + i;
       }
   }
-  if (kernel == 2)
-    return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, shape, stream);
   // (a shape given by the caller for the wide kernel may carry a cut of K in front: cuts * 10000000 + shape)
   if (kernel == 4)
-    return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, act, algo == 4 ? shape % 10000000 : 0,
+    return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, activated ? activated : act, algo == 4 ? shape % 10000000 : 0,
                      algo == 4 ? shape / 10000000 : 1, workspace, ws_bytes, stream, planes_left);
-  if (kernel == 3)
-    return gemm_tiled(A, lda, W, C, c_dtype, ldc, M, N, K, epilogue, act, cap, shape, workspace, ws_bytes, stream);
-  return gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, stream);
+  int rc;
+  if (kernel == 2)
+    rc = gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, shape, stream);
+  else if (kernel == 3)
+    rc = gemm_tiled(A, lda, W, C, c_dtype, ldc, M, N, K, epilogue, act, cap, shape, workspace, ws_bytes, stream);
+  else
+    rc = gemm_generic(A, a_dtype, lda, W, W2, w_dtype, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, stream);
+  if (rc == 0 && activated) rc = apply_activation(C, c_dtype, ldc, M, N, activated - 1, stream);
+  return rc;
 }
 
 extern "C" int sa_gemm(const void* A, int a_dtype, int64_t lda, const void* W, const void* W2, int w_dtype, void* C,

@@ -373,7 +373,7 @@ def decode_slots(positions: torch.Tensor, token_seq: torch.Tensor, block_table: 
 
 # --------------------------------------------------------------------------- matrix products
 
-EPILOGUE_NONE, EPILOGUE_GATED, EPILOGUE_SOFT_CAP = 0, 1, 2
+EPILOGUE_NONE, EPILOGUE_GATED, EPILOGUE_SOFT_CAP, EPILOGUE_ACTIVATED = 0, 1, 2, 3
 #: activations of the gated epilogue (simply_amd/csrc/activations.h); the epilogue argument is 1 + 16 * activation
 ACT_GELU_TANH, ACT_SILU, ACT_SQUARED_RELU = 0, 1, 2
 
@@ -410,9 +410,10 @@ def workspace_uses(device) -> int:
 def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor | TiledWeight | None" = None,
          soft_cap: float | None = None, out_dtype: torch.dtype | None = None, out: torch.Tensor | None = None,
          algo: int = ALGO_AUTO, shape: int = 0, activation: int = ACT_GELU_TANH,
-         defer_sum: bool = False) -> "torch.Tensor | PartialSums":
+         defer_sum: bool = False, activate: int | None = None) -> "torch.Tensor | PartialSums":
     """a[M, K] . w[N, K]^T.  With w2 (row-major weights) or a paired `TiledWeight`: act(a.wg^T) * (a.wu^T) with
-    the activation of that code.  With soft_cap: cap * tanh(. / cap).  w is a row-major tensor or a `TiledWeight`.
+    the activation of that code.  With soft_cap: cap * tanh(. / cap).  With activate (an activation code): act(a.w^T),
+    the product rounded to the output type first.  w is a row-major tensor or a `TiledWeight`.
     defer_sum: where the product is computed in cuts of K, leave their sum to the caller: the result is then a
     `PartialSums` (else the tensor as always)."""
     packed = isinstance(w, TiledWeight)
@@ -444,6 +445,10 @@ def gemm(a: torch.Tensor, w: "torch.Tensor | TiledWeight", *, w2: "torch.Tensor 
         epi = _gated(activation)
     elif soft_cap:
         epi, cap = EPILOGUE_SOFT_CAP, float(soft_cap)
+    if activate is not None:
+        if epi != EPILOGUE_NONE or defer_sum:
+            raise KernelError("gemm: an activation of the product combines with no other epilogue and no deferred sum")
+        epi = _gated(activate) - EPILOGUE_GATED + EPILOGUE_ACTIVATED
     if out is None:
         out = torch.empty((M, N), dtype=out_dtype or a.dtype, device=a.device)
     if tuple(out.shape) != (M, N):

@@ -36,7 +36,7 @@ class Dense(FeedForward):
         self.down_proj = as_product_weight(tensors["down_proj"])
 
     def forward(self, x: torch.Tensor, ctx=None, defer_sum=False) -> torch.Tensor:
-        z = ops.activation_(ops.gemm(x, self.up_proj), self.activation_code)
+        z = ops.gemm(x, self.up_proj, activate=self.activation_code)   # (the activation is the product's epilogue)
         return ops.gemm(z, self.down_proj, defer_sum=defer_sum)
 
 

@@ -28,6 +28,11 @@ def test_kernel(body, dtype):
     body(ops, DEV, dtype)
 
 
+@pytest.mark.parametrize("dtype, tiled", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+def test_activated_product(dtype, tiled):
+    mech.activated_product(ops, DEV, dtype, tiled)
+
+
 def test_partial_rotary_into_tiled_pages():
     """Pages of 16 keys of a size that is a multiple of 32 are stored in operand blocks: the same test, that layout."""
     mech.partial_rotary_norm_and_pages(ops, DEV, torch.bfloat16, page_size=16)

@@ -77,6 +77,10 @@ def test_reference_of_a_kernel(body):
     body(torch_ops, CPU, torch.float32)
 
 
+def test_reference_of_the_activated_product():
+    mech.activated_product(torch_ops, CPU, torch.float32)
+
+
 def test_reference_of_the_recurrence():
     mech.delta_rule_steps(torch_ops, CPU)
 

@@ -118,7 +118,8 @@ def squared_relu(x):
 ACTIVATIONS = (gelu_tanh, silu, squared_relu)   # by the kernels' activation codes
 
 
-def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shape=0, activation=0, defer_sum=False):
+def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shape=0, activation=0, defer_sum=False,
+         activate=None):
     # (defer_sum: the kernels may leave a sum to the caller; this stand-in never cuts a product)
     out_dtype = out_dtype or a.dtype
     if getattr(w, "paired", False):
@@ -130,6 +131,8 @@ def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shap
         c = ACTIVATIONS[activation](_f(c.to(out_dtype))) * _f(up.to(out_dtype))
     elif soft_cap:
         c = soft_cap * torch.tanh(c / soft_cap)
+    elif activate is not None:
+        c = ACTIVATIONS[activate](_f(c.to(out_dtype)))
     c = c.to(out_dtype)
     if out is not None:
         out.copy_(c)

@@ -70,6 +70,21 @@ def activation(o, device, dtype):
     close(got, plain.gelu_tanh(x.double()), tol_of(dtype))
 
 
+def activated_product(o, device, dtype, tiled=False):
+    """relu(x W^T)^2 as one call, at row counts that the different product kernels take (a handful, a few hundred
+    with the inner dimension cut over workgroups, thousands with the activation in the kernel's epilogue)."""
+    from simply_amd.parts.base import as_product_weight
+
+    K, N = 256, 384
+    w = rand((N, K), 20, 0.1).to(dtype)
+    wd = as_product_weight(w.to(device)) if tiled else w.to(device)
+    for M in (3, 40, 300, 2100):
+        x = rand((M, K), 21 + M).to(dtype)
+        want = plain.squared_relu((x.double() @ w.double().T).to(dtype).double())
+        got = o.gemm(x.to(device), wd, activate=registry.ACTIVATIONS.get("squared_relu"))
+        close(got, want, 2e-5 if dtype == torch.float32 else 3e-2, f"{M} rows")
+
+
 def partial_rotary_norm_and_pages(o, device, dtype, page_size=4):
     """Queries and keys: rotation of the first dimensions, then unit RMS; values mixed; pages written where the slot
     mapping says.  Positions far from 0 and a page's last and first place are among them."""
