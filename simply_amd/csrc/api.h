@@ -322,7 +322,8 @@ int sa_short_conv_silu(const void* x, int x_dtype, int64_t x_stride, const void*
 int sa_delta_prepare(float* qkv, int T, int C, int G, int dk, const void* ab, int ab_dtype, int64_t ab_stride,
                      const void* a_log, const void* dt_bias, int vec_dtype, int H, float* gates, hipStream_t stream);
 
-// The gated delta rule over each request's tokens, from and into state[slot] [H][dk][dv] float32: per head
+// The gated delta rule over each request's tokens, from and into state[slot] float32, per head the matrix S [dk, dv]
+// stored column by column ([H][dv][dk]): per head
 // S <- g S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.  Value head h reads q/k head h / (H / G).
 int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, const float* gates, int H, float* state,
                   int64_t state_stride, const int* seq_meta, int num_seqs, float* out, hipStream_t stream);

@@ -149,12 +149,13 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
   const int col = blockIdx.z * COLS + tid / LPC, part = tid % LPC;
   const bool live = col < dv;
   const int qk_head = h / (H / G);
-  float* S = state + static_cast<size_t>(slot) * state_stride + static_cast<size_t>(h) * dk * dv;   // [dk][dv]
+  // a head's state is kept column by column, [dv][dk]: the lanes that share a column read neighbouring words
+  float* S = state + static_cast<size_t>(slot) * state_stride + static_cast<size_t>(h) * dk * dv;
   float s[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = r * LPC + part;
-    s[r] = (live && i < dk) ? S[static_cast<size_t>(i) * dv + col] : 0.f;
+    s[r] = (live && i < dk) ? S[static_cast<size_t>(col) * dk + i] : 0.f;
   }
   const int v_at = 2 * G * dk + h * dv;
   // A tile's q, k, v and gates are asked for a tile ahead, into registers, and put into LDS when the tile's turn
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     const int i = r * LPC + part;
-    if (live && i < dk) S[static_cast<size_t>(i) * dv + col] = s[r];
+    if (live && i < dk) S[static_cast<size_t>(col) * dk + i] = s[r];
   }
 }
 

@@ -897,7 +897,7 @@ def delta_prepare(qkv: torch.Tensor, ab: torch.Tensor, a_log: torch.Tensor, dt_b
 def delta_rule(qkv: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int,
                num_heads: int, num_qk_heads: int, key_dim: int, value_dim: int) -> torch.Tensor:
     """The gated delta rule along each request's tokens, from and into state [slots, >= H * dk * dv] float32 (per
-    slot [H][dk][dv]).  qkv float32 [T, C] as `delta_prepare` left it, gates [T, 2 H].  Returns float32 [T, H * dv]."""
+    slot and head the matrix S [dk, dv], stored column by column: [H][dv][dk]).  qkv float32 [T, C] as `delta_prepare` left it, gates [T, 2 H].  Returns float32 [T, H * dv]."""
     _dev(qkv, gates, state, seq_meta)
     T, C = qkv.shape
     H, G, dk, dv = num_heads, num_qk_heads, key_dim, value_dim

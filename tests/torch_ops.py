@@ -337,7 +337,7 @@ def delta_rule(qkv, gates, state, seq_meta, num_seqs, num_heads, num_qk_heads, k
     out = torch.empty((T, H * dv), dtype=torch.float32, device=qkv.device)
     x, gt = _f(qkv), _f(gates)
     for slot, first, count, _ in seq_meta[:num_seqs].tolist():
-        S = _f(state[slot, :H * dk * dv]).reshape(H, dk, dv).clone()
+        S = _f(state[slot, :H * dk * dv]).reshape(H, dv, dk).transpose(1, 2).clone()   # stored column by column
         for t in range(first, first + count):
             for h in range(H):
                 j = h // (H // G)
@@ -347,7 +347,7 @@ def delta_rule(qkv, gates, state, seq_meta, num_seqs, num_heads, num_qk_heads, k
                 u = gt[t, h] * (v - S[h].T @ k)
                 S[h] = S[h] + torch.outer(k, u)
                 out[t, h * dv:(h + 1) * dv] = (S[h].T @ q).to(torch.float32)
-        state[slot, :H * dk * dv] = S.reshape(-1).to(torch.float32)
+        state[slot, :H * dk * dv] = S.transpose(1, 2).reshape(-1).to(torch.float32)
     return out
 
 

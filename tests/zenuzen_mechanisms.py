@@ -215,7 +215,7 @@ def delta_rule_steps(o, device):
         got.append(o.delta_rule(part, gates, state, meta, 1, H, G, dk, dv).cpu())
         at += c
     close(torch.cat(got), want.reshape(T, H * dv), 3e-5, "outputs")
-    close(state[1, :H * dk * dv].view(H, dk, dv), S, 3e-5, "state")
+    close(state[1, :H * dk * dv].view(H, dv, dk).transpose(1, 2), S, 3e-5, "state (stored column by column)")
     assert float(state[0].abs().max()) == 0.0 and float(state[2].abs().max()) == 0.0
 
 
