@@ -47,6 +47,10 @@ def test_attention_part(dtype):
     mech.attention_part(DEV, dtype)
 
 
+def test_sink_attention_kernels_on_the_matrix_cores():
+    mech.sink_attention_on_the_matrix_cores(DEV)
+
+
 def test_attention_part_on_the_matrix_cores():
     """Values of the keys' size (64) in pages of 16 keys, bfloat16: the MFMA kernels run, few rows a request and
     portions of prompts, with their key ranges merged, the sinks in every sum and the scores' factor in the queries."""

@@ -132,7 +132,7 @@ def sink_attention_far_key(o, device, dtype, page_size=16):
     T, H, K, dk, dv, scale = 300, 4, 2, 24, 12, 0.6
     q, k, v = rand((T, H, dk), 10), rand((T, K, dk), 11), rand((T, K, dv), 12)
     sink = torch.tensor([2.0, -1.0, 0.5, 4.0], dtype=torch.float64)
-    for far, asker, head in ((15, 299, 0), (0, 250, 3), (16, 17, 1)):
+    for far, asker, head in ((15, 299, 0), (0, 250, 3), (16, 17, 1), (63, 100, 2), (64, 31 + 64, 0)):
         k[far, head // 2] = q[asker, head] * (25.0 / (q[asker, head] ** 2).sum())   # a score of 25 * scale, far above the others
     qd, kd, vd = q.to(dtype), k.to(dtype), v.to(dtype)
     want = plain.sink_softmax_attention(qd.double(), kd.double(), vd.double(), sink.to(dtype).double(), scale)
@@ -152,7 +152,7 @@ def sink_attention_far_key(o, device, dtype, page_size=16):
         krows[page, :, off] = kd[t]
         v_pages[page, :, :, off] = vd[t]
     k_pages = torch_ops.rows_as_stored_keys(krows)
-    rows = torch.tensor([299, 250, 17, 0, 1, 15, 16, 31, 32, 100], dtype=torch.long)
+    rows = torch.tensor([299, 250, 17, 0, 1, 15, 16, 31, 32, 100, 95, 63, 64], dtype=torch.long)
     got = o.paged_attention_sink(qd[rows].reshape(len(rows), H * dk).contiguous().to(device), k_pages.to(device),
                                  v_pages.to(device), table.to(device), torch.ones(len(rows), dtype=torch.int32, device=device),
                                  rows.to(torch.int32).to(device), H, scale=scale, sinks=sink.to(dtype).to(device))
@@ -161,6 +161,60 @@ def sink_attention_far_key(o, device, dtype, page_size=16):
     first = got[3].double().cpu().view(H, dv)
     share = 1.0 / (1.0 + torch.exp(sink.to(dtype).double() - scale * (qd[0].double() * kd[0].double().repeat_interleave(2, 0)).sum(-1)))
     close(first, vd[0].double().repeat_interleave(2, 0) * share[:, None], tol_of(dtype), "the first token and the sink")
+
+
+def sink_attention_on_the_matrix_cores(device):
+    """The bfloat16 MFMA kernels with sinks: single tokens (their keys cut into ranges that a second kernel merges)
+    and a portion of a prompt, with far keys that stand out (at position 0, at a page's last and first place, at the
+    edge of a tile of 32 keys) among a thousand, and one large sink."""
+    import torch_ops
+    from simply_amd.engine.context import StepContext
+    from simply_amd.kernels import ops
+
+    T, H, K, d, scale, P = 1000, 8, 2, 64, 0.3, 16
+    dtype = torch.bfloat16
+    q, k, v = rand((T, H, d), 50), rand((T, K, d), 51), rand((T, K, d), 52)
+    sink = torch.tensor([6.0, -1.0, 0.5, 4.0, 0.0, 2.0, -3.0, 8.0], dtype=torch.float64)
+    for far, asker, head in ((0, 999, 0), (15, 990, 3), (16, 999, 5), (31, 700, 7), (32, 969, 1), (511, 998, 6)):
+        k[far, head // 4] = q[asker, head] * (40.0 / (q[asker, head] ** 2).sum())
+    qd, kd, vd = q.to(dtype), k.to(dtype), v.to(dtype)
+    want = plain.sink_softmax_attention(qd.double(), kd.double(), vd.double(), sink, scale)
+    n_pages = -(-T // P)
+    order = torch.randperm(n_pages + 5, generator=torch.Generator().manual_seed(2))[:n_pages]
+    table = torch.full((2, n_pages), -1, dtype=torch.int32)
+    table[1] = order.to(torch.int32)
+    krows = torch.zeros((n_pages + 5, K, P, d), dtype=dtype)
+    v_pages = torch.zeros((n_pages + 5, K, d, P), dtype=dtype)
+    for t in range(T):
+        krows[int(order[t // P]), :, t % P] = kd[t]
+        v_pages[int(order[t // P]), :, :, t % P] = vd[t]
+    k_pages = torch_ops.rows_as_stored_keys(krows).to(device)
+    v_pages, table = v_pages.to(device), table.to(device)
+    sinks = sink.float().to(device)
+    # (these kernels have no factor on the scores: the queries carry it)
+    qs = (qd.double() * scale).to(dtype).reshape(T, H * d).to(device)
+    # single tokens: every row a request of its own at its position
+    rows = [999, 990, 700, 969, 998, 0, 15, 16, 31, 32, 33, 512]
+    meta = torch.tensor([[1, i, 1, r] for i, r in enumerate(rows)], dtype=torch.int32, device=device)
+    out = torch.zeros((len(rows), H * d), dtype=dtype, device=device)
+    ops.paged_attention_decode(qs[rows].contiguous(), k_pages, v_pages, table, meta, 0, len(rows), H, window=None,
+                               soft_cap=None, max_kv_len=T, max_q_len=1, out=out, sinks=sinks)
+    close(out, want[rows].reshape(len(rows), H * d), 3e-2, "single tokens")
+    # the last 299 tokens as one portion of a prompt
+    first = T - 299
+    ctx = StepContext(dtype=dtype, num_tokens=299, positions=torch.arange(first, T, dtype=torch.int32, device=device),
+                      token_seq=torch.ones(299, dtype=torch.int32, device=device),
+                      seq_meta=torch.tensor([[1, 0, 299, first]], dtype=torch.int32, device=device), groups={},
+                      request_ids=["r"], seq_slots=[1], seq_starts=[first], q_lens=[299], cu_q_lens=[0, 299])
+    units, few, many, max_q = ctx.attention_units(16 // (H // K), ops.prefill_units_per_group())
+    assert few == 0 and many > 0
+    out = torch.zeros((299, H * d), dtype=dtype, device=device)
+    ops.paged_attention_prefill(qs[first:].contiguous(), k_pages, v_pages, table, units, 0, many, H, window=None,
+                                soft_cap=None, max_kv_len=T, max_q_len=max_q, out=out, sinks=sinks)
+    close(out, want[first:].reshape(299, H * d), 3e-2, "a portion")
+    # the sinks matter: without them the answer is another one
+    without = plain.sink_softmax_attention(qd.double(), kd.double(), vd.double(), sink - 50.0, scale)
+    assert float((without[first:] - want[first:]).abs().max()) > 0.3
 
 
 def short_convolution(o, device, dtype):
