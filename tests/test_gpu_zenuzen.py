@@ -83,6 +83,18 @@ def test_pages_of_sixteen_keys(tmp_path):
     cases.long_decoding(tmp_path / "l", DEV, "aligned", "bfloat16", steps=150, page_size=16)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_drawn_configurations(tmp_path, seed):
+    """Configurations drawn at random (sizes, head counts, layer order, feed-forwards, value mixing, rotation, taps):
+    unequal requests in portions beside single tokens, in 32-bit against the plain implementation."""
+    cases.drawn_configuration_runs(tmp_path, DEV, seed, "float32")
+
+
+@pytest.mark.parametrize("seed", [3, 7, 11])
+def test_drawn_configurations_bfloat16(tmp_path, seed):
+    cases.drawn_configuration_runs(tmp_path, DEV, seed, "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding(tmp_path, dtype):
     cases.long_decoding(tmp_path, DEV, "mixed", dtype, steps=150, page_size=16)

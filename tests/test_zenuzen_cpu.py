@@ -104,6 +104,12 @@ def test_batches_match_alone(tmp_path, cpu_ops, name):
     cases.batches_match_alone(tmp_path, CPU, name)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_drawn_configurations(tmp_path, cpu_ops, seed):
+    config_from_dict(cases.drawn_config(seed))    # (every drawn configuration is a valid one)
+    cases.drawn_configuration_runs(tmp_path, CPU, seed)
+
+
 def test_long_decoding(tmp_path, cpu_ops):
     cases.long_decoding(tmp_path, CPU, "mixed", steps=70, page_size=4)
 

@@ -68,6 +68,63 @@ CONFIGS = {"mixed": (MIXED, 11), "only_delta": (ONLY_DELTA, 12), "only_attention
            "aligned": (ALIGNED, 14)}
 
 
+def drawn_config(seed: int) -> dict:
+    """A configuration drawn at random: sizes, head counts, the order of the layers, which layers have a
+    feed-forward, which mix values, how much of a head is rotated, taps, multiplier and eps."""
+    import random
+
+    r = random.Random(seed)
+    width = r.choice([24, 40, 56, 64, 96])
+    layers = []
+    mix_shape = (r.choice([1, 2]), r.choice([8, 12, 20, 32]))      # layers that mix values agree in these
+    for _ in range(r.randint(2, 6)):
+        mlp = r.choice([None, None, r.choice([32, 48, 100])])
+        if r.random() < 0.45:
+            v_mix = r.random() < 0.6
+            kv, vdim = mix_shape if v_mix else (r.choice([1, 2, 3]), r.choice([4, 8, 16, 24]))
+            dim = r.choice([8, 12, 16, 32, 48])
+            rot = r.choice([None, (r.choice([2, 4, dim]), r.choice([100.0, 10000.0, 1e6]))])
+            layers.append(attention(kv * r.choice([1, 2, 3, 4]), kv, dim, vdim, r.choice([0.2, 0.5, dim ** -0.5]), rot=rot,
+                                    v_mix=v_mix, mlp=mlp))
+        else:
+            g = r.choice([1, 2, 3])
+            layers.append(delta(g * r.choice([1, 2, 4]), g, r.choice([4, 8, 16, 24, 40, 72]), r.choice([4, 8, 20, 70]),
+                                r.choice([1, 2, 3, 4, 5, 8]), mlp=mlp))
+    return config(r.choice([50, 97, 130, 300]), width, r.choice([0.3, 0.7, 1.0, 1.4]), r.choice([1e-6, 1e-5, 1e-3]), layers)
+
+
+def drawn_configuration_runs(tmp_path, device, seed: int, dtype="float32"):
+    """A drawn configuration, three requests of unequal length in portions beside single tokens, in a tight pool."""
+    d = write_random_model(config_from_dict(drawn_config(seed)), str(tmp_path / f"m{seed}"), seed, torch.float32, std=0.3,
+                           norm_std=0.4)
+    w, cfg = plain_weights(d, dtype)
+    toks = {r: random_tokens(n, cfg["vocab"], seed * 10 + i) for i, (r, n) in enumerate((("a", 41), ("b", 13), ("c", 26)))}
+    want = {r: plain.forward(w, cfg, t) for r, t in toks.items()}
+    ex = make_executor(d, device, dtype, page_size=4, num_pages=24, batch=2, max_len=44, poison=True)
+    schedule = [[("a", 9), ("b", 2)], [("a", 1), ("b", 7)], [("a", 17), ("b", 1)], [("a", 2), ("b", 3)],   # b ends
+                [("a", 1), ("c", 20)], [("a", 11), ("c", 1)], [("c", 2)], [("c", 3)]]
+    done = {r: 0 for r in toks}
+    got = {r: [] for r in toks}
+    for step in schedule:
+        entries = []
+        for r, n in step:
+            if not ex.has_request(r):
+                ex.add_request(r)
+            entries.append(StepEntry(r, toks[r][done[r]:done[r] + n], list(range(n))))
+        logits = ex.step(entries).cpu()
+        at = 0
+        for r, n in step:
+            got[r].append(logits[at:at + n])
+            at += n
+            done[r] += n
+            if done[r] == len(toks[r]):
+                ex.finish_request(r)
+        ex.cache.check()
+    for r in toks:
+        assert done[r] == len(toks[r])
+        assert_close_logits(torch.cat(got[r]), want[r], dtype, (seed, r))
+
+
 def write_model(name: str, out_dir: str, dtype=torch.float32, std: float = 0.25, norm_std: float = 0.5) -> str:
     """Writes the configuration with random weights through the framework's random-weights mode.  Norm weights,
     sinks, decays and the mixing factor are drawn around 0 with norm_std."""
