@@ -317,23 +317,16 @@ int sa_short_conv_silu(const void* x, int x_dtype, int64_t x_stride, const void*
                        int C, int update_tails, hipStream_t stream);
 
 // In place on qkv [T, C] float32 = [G q heads | G k heads | values]: q and k heads to unit length
-// (x / sqrt(sum(x^2) + 1e-6)), q also times dk^(-1/2).  gates [T, 3 H] receives beta = sigmoid(b),
-// g = exp(-exp(a_log) * softplus(a + dt_bias)) and ln g from ab [T, a (H) | b (H)].
+// (x / sqrt(sum(x^2) + 1e-6)), q also times dk^(-1/2).  gates [T, 2 H] receives beta = sigmoid(b) and
+// g = exp(-exp(a_log) * softplus(a + dt_bias)) from ab [T, a (H) | b (H)].
 int sa_delta_prepare(float* qkv, int T, int C, int G, int dk, const void* ab, int ab_dtype, int64_t ab_stride,
                      const void* a_log, const void* dt_bias, int vec_dtype, int H, float* gates, hipStream_t stream);
 
 // The gated delta rule over each request's tokens, from and into state[slot] float32, per head the matrix S [dk, dv]
 // stored column by column ([H][dv][dk]): per head
 // S <- g S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.  Value head h reads q/k head h / (H / G).
-// Requests that bring at least sa_delta_rule_chunk_threshold(dk) tokens (0: none, at this key size) are worked
-// through in chunks of 32 tokens by two kernels (the factors of all chunks at once, then the state's walk from chunk
-// to chunk) if `scratch` holds sa_delta_rule_scratch_words(num_seqs, max_q_len, H) floats; the others, and all of
-// them without scratch memory, token by token.  min_q_len, max_q_len: the fewest and the most tokens of a request.
-int sa_delta_rule_chunk_threshold(int dk);
-int64_t sa_delta_rule_scratch_words(int num_seqs, int max_q_len, int H);
 int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, const float* gates, int H, float* state,
-                  int64_t state_stride, const int* seq_meta, int num_seqs, int min_q_len, int max_q_len, float* scratch,
-                  int64_t scratch_words, float* out, hipStream_t stream);
+                  int64_t state_stride, const int* seq_meta, int num_seqs, float* out, hipStream_t stream);
 
 // sa_paged_attention_decode and sa_paged_attention_prefill for softmax sums that hold one more term per query head,
 // exp(sinks[h]) (float32 [H]; null: none), without a value.

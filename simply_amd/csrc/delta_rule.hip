@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kWave) void conv_tail_update_kernel(const void* __r
 
 // Per (token, unit): units 0 .. 2 G - 1 are the q and k heads of qkv [T, C] (q heads first), each made a unit vector
 // x / sqrt(sum(x^2) + 1e-6), the queries also times size^(-1/2); unit 2 G computes, for every value head h,
-// beta = sigmoid(b), g = exp(-exp(A_log) * softplus(a + dt_bias)) and ln g into gates [T, 3 H] (in this order).
+// beta = sigmoid(b) and g = exp(-exp(A_log) * softplus(a + dt_bias)) into gates [T, 2 H] (beta first).
 __global__ __launch_bounds__(kWave) void delta_prepare_kernel(float* __restrict__ qkv, int C, int G, int dk,
                                                               const void* __restrict__ ab, int ab_dtype,
                                                               int64_t ab_stride, const void* __restrict__ a_log,
@@ -98,10 +98,8 @@ __global__ __launch_bounds__(kWave) void delta_prepare_kernel(float* __restrict_
     const float b = load_f(ab, ab_dtype, static_cast<size_t>(t) * ab_stride + H + h);
     const float z = a + load_f(dt_bias, vec_dtype, h);
     const float sp = z > 30.f ? z : log1pf(expf(z));
-    const float lg = -expf(load_f(a_log, vec_dtype, h)) * sp;
-    gates[static_cast<size_t>(t) * 3 * H + h] = 1.f / (1.f + expf(-b));
-    gates[static_cast<size_t>(t) * 3 * H + H + h] = expf(lg);
-    gates[static_cast<size_t>(t) * 3 * H + 2 * H + h] = lg;
+    gates[static_cast<size_t>(t) * 2 * H + h] = 1.f / (1.f + expf(-b));
+    gates[static_cast<size_t>(t) * 2 * H + H + h] = expf(-expf(load_f(a_log, vec_dtype, h)) * sp);
   }
 }
 
@@ -114,6 +112,7 @@ __global__ __launch_bounds__(kWave) void delta_prepare_kernel(float* __restrict_
 // per token, and the instructions that one wave issues for it, are what bound a prompt's time (tokens follow one
 // another, and a head's columns are all the waves there are): 16 or 32 lanes per column keep both short where a
 // column has 64 rows or more.
+constexpr int kRuleTokens = 16;
 template <int LPC>
 __device__ __forceinline__ float lanes_sum(float v) {
   v += lane_exchange<0xB1>(v);   // quad_perm [1, 0, 3, 2]
@@ -135,19 +134,17 @@ __device__ __forceinline__ float lanes_sum(float v) {
   return v;
 }
 
-template <int DK, int LPC, int kRuleTokens>
+template <int DK, int LPC>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ qkv, int C, int G, int dk, int dv,
                                                          const float* __restrict__ gates, int H,
                                                          float* __restrict__ state, int64_t state_stride,
-                                                         const int* __restrict__ seq_meta, float* __restrict__ out,
-                                                         int max_count) {
+                                                         const int* __restrict__ seq_meta, float* __restrict__ out) {
   constexpr int R = DK / LPC, COLS = 256 / LPC;
   static_assert(R % 4 == 0 || R < 4, "rows per lane come in fours");
   constexpr int NACC = R < 4 ? 1 : 4;
   __shared__ float qs[kRuleTokens][DK], ks[kRuleTokens][DK], vs[kRuleTokens][COLS], bg[kRuleTokens][2];
   const int* meta = seq_meta + 4 * blockIdx.x;
   const int slot = meta[0], first = meta[1], count = meta[2];
-  if (count >= max_count) return;   // (the chunked kernels take the requests with many tokens)
   const int h = blockIdx.y, tid = threadIdx.x;
   const int col = blockIdx.z * COLS + tid / LPC, part = tid % LPC;
   const bool live = col < dv;
@@ -181,7 +178,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
       const bool ok = idx < kRuleTokens * COLS && j < tn && c < dv;
       pv[i] = ok ? qkv[static_cast<size_t>(first + t0 + j) * C + v_at + c] : 0.f;
     }
-    pg = tid < 2 * tn ? gates[static_cast<size_t>(first + t0 + tid / 2) * 3 * H + (tid % 2) * H + h] : 0.f;
+    pg = tid < 2 * tn ? gates[static_cast<size_t>(first + t0 + tid / 2) * 2 * H + (tid % 2) * H + h] : 0.f;
   };
   if (count > 0) fetch(0);
   for (int t0 = 0; t0 < count; t0 += kRuleTokens) {
@@ -224,8 +221,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
         s[r] *= x.g;
         d[r % NACC] = fmaf(s[r], x.k[r], d[r % NACC]);
       }
-      float dot = d[0];
-      if (NACC == 4) dot = (d[0] + d[NACC > 1 ? 1 : 0]) + (d[NACC > 2 ? 2 : 0] + d[NACC > 3 ? 3 : 0]);
+      float dot = NACC == 4 ? (d[0] + d[1]) + (d[2] + d[3]) : d[0];
       dot = lanes_sum<LPC>(dot);
       const float u = x.beta * (x.v - dot);
 #pragma unroll
@@ -235,8 +231,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
         s[r] = fmaf(x.k[r], u, s[r]);
         d[r % NACC] = fmaf(s[r], x.q[r], d[r % NACC]);
       }
-      float o = d[0];
-      if (NACC == 4) o = (d[0] + d[NACC > 1 ? 1 : 0]) + (d[NACC > 2 ? 2 : 0] + d[NACC > 3 ? 3 : 0]);
+      float o = NACC == 4 ? (d[0] + d[1]) + (d[2] + d[3]) : d[0];
       o = lanes_sum<LPC>(o);
       if (live && part == 0)
         out[static_cast<size_t>(first + t0 + j) * (static_cast<size_t>(H) * dv) + static_cast<size_t>(h) * dv + col] = o;
@@ -256,187 +251,6 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
   for (int r = 0; r < R; ++r) {
     const int i = r * LPC + part;
     if (live && i < dk) S[static_cast<size_t>(col) * dk + i] = s[r];
-  }
-}
-
-
-// ------------------------------------------------------------------ the same rule, a chunk of 32 tokens at a time
-// For requests that bring many tokens.  Within a chunk, with L_t = ln g_1 + ... + ln g_t counted from the chunk's
-// start, S0 the state before the chunk and e(t, i) = exp(L_t - L_i):
-//
-//   u_t = beta_t (v_t - exp(L_t) S0^T k_t - sum_{i<t} e(t, i) (k_t . k_i) u_i)
-//   o_t = exp(L_t) S0^T q_t + sum_{i<=t} e(t, i) (q_t . k_i) u_i
-//   S   = exp(L_C) S0 + sum_t e(C, t) k_t u_t^T
-//
-// so with A[t][i] = beta_t e(t, i) (k_t . k_i) below the diagonal, U = (I + A)^-1 B for B_t = beta_t (v_t -
-// exp(L_t) S0^T k_t).  The first kernel computes, for every chunk and head at once, T = (I + A)^-1 and
-// P[t][i] = e(t, i) (q_t . k_i) (neither depends on the state); the second walks a request's chunks in order with a
-// block of the state's columns in LDS and does, per chunk, the products with S0, U = T B, the outputs and the new
-// state: sums of 32 or of the key size per element, no sum across lanes, all 32-bit.  The order of the sums differs
-// from the token-by-token kernel's (rounding only).  A chunk's factors lie in `scratch` as [T 32x32][P 32x32]
-// [exp(L_t) 32][e(C, t) 32][beta 32] per (request, chunk, head); tokens beyond a request's last count as beta = 0,
-// g = 1, k = q = 0.
-constexpr int kChunk = 32;
-constexpr int kChunkWords = 2 * kChunk * kChunk + 3 * kChunk;
-
-template <int DK>
-__global__ __launch_bounds__(256) void delta_chunk_factors_kernel(const float* __restrict__ qkv, int C, int G, int dk,
-                                                                  const float* __restrict__ gates, int H,
-                                                                  const int* __restrict__ seq_meta, int min_count,
-                                                                  float* __restrict__ scratch, int max_chunks) {
-  constexpr int LD = DK + 1;
-  __shared__ float ks[kChunk][LD], qs[kChunk][LD];
-  __shared__ float Am[kChunk][kChunk + 1], Tm[kChunk][kChunk + 1], Lc[kChunk], bt[kChunk];
-  const int n = blockIdx.x, s = blockIdx.y, h = blockIdx.z, tid = threadIdx.x;
-  const int* meta = seq_meta + 4 * s;
-  const int first = meta[1], count = meta[2];
-  const int t0 = n * kChunk;
-  if (count < min_count || t0 >= count) return;
-  const int tn = count - t0 < kChunk ? count - t0 : kChunk;
-  const int qk_head = h / (H / G);
-  for (int idx = tid; idx < kChunk * DK; idx += 256) {
-    const int j = idx / DK, d = idx % DK;
-    const bool ok = j < tn && d < dk;
-    const float* row = qkv + static_cast<size_t>(first + t0 + (ok ? j : 0)) * C;
-    ks[j][d] = ok ? row[(G + qk_head) * dk + d] : 0.f;
-    qs[j][d] = ok ? row[qk_head * dk + d] : 0.f;
-  }
-  if (tid < kChunk) {
-    const size_t g_at = static_cast<size_t>(first + t0 + tid) * 3 * H + h;
-    bt[tid] = tid < tn ? gates[g_at] : 0.f;
-    Lc[tid] = tid < tn ? gates[g_at + 2 * H] : 0.f;
-  }
-  __syncthreads();
-  if (tid == 0)
-    for (int t = 1; t < kChunk; ++t) Lc[t] += Lc[t - 1];
-  __syncthreads();
-  float* out = scratch + ((static_cast<size_t>(s) * max_chunks + n) * H + h) * kChunkWords;
-  for (int idx = tid; idx < kChunk * kChunk; idx += 256) {
-    const int t = idx / kChunk, i = idx % kChunk;
-    float a = 0.f, p = 0.f;
-    if (i <= t) {
-      float dk_[4] = {0.f, 0.f, 0.f, 0.f}, dq_[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-      for (int d = 0; d < DK; ++d) {
-        dk_[d % 4] = fmaf(ks[t][d], ks[i][d], dk_[d % 4]);
-        dq_[d % 4] = fmaf(qs[t][d], ks[i][d], dq_[d % 4]);
-      }
-      const float e = expf(Lc[t] - Lc[i]);
-      p = e * ((dq_[0] + dq_[1]) + (dq_[2] + dq_[3]));
-      if (i < t) a = bt[t] * e * ((dk_[0] + dk_[1]) + (dk_[2] + dk_[3]));
-    }
-    Am[t][i] = a;
-    out[kChunk * kChunk + idx] = p;
-  }
-  __syncthreads();
-  if (tid < kChunk) {   // column tid of (I + A)^-1, from the diagonal down
-    const int j = tid;
-    for (int t = 0; t < kChunk; ++t) {
-      float v = t == j ? 1.f : 0.f;
-      for (int i = j; i < t; ++i) v = fmaf(-Am[t][i], Tm[i][j], v);
-      Tm[t][j] = v;
-    }
-    out[2 * kChunk * kChunk + tid] = expf(Lc[tid]);
-    out[2 * kChunk * kChunk + kChunk + tid] = expf(Lc[kChunk - 1] - Lc[tid]);
-    out[2 * kChunk * kChunk + 2 * kChunk + tid] = bt[tid];
-  }
-  __syncthreads();
-  for (int idx = tid; idx < kChunk * kChunk; idx += 256) out[idx] = Tm[idx / kChunk][idx % kChunk];
-}
-
-template <int DK>
-__global__ __launch_bounds__(256) void delta_chunk_scan_kernel(const float* __restrict__ qkv, int C, int G, int dk, int dv,
-                                                               int H, float* __restrict__ state, int64_t state_stride,
-                                                               const int* __restrict__ seq_meta, int min_count,
-                                                               const float* __restrict__ scratch, int max_chunks,
-                                                               float* __restrict__ out) {
-  constexpr int NC = 8, LD = DK + 4;   // columns of the state per workgroup; rows of 16-byte pieces
-  __shared__ __attribute__((aligned(16))) float ks[kChunk][LD];
-  __shared__ __attribute__((aligned(16))) float qs[kChunk][LD];
-  __shared__ __attribute__((aligned(16))) float Ss[NC][LD];   // the columns, each with its rows side by side
-  __shared__ float Tm[kChunk][kChunk + 1], Pm[kChunk][kChunk + 1];
-  __shared__ float vs[kChunk][NC], Bm[kChunk][NC], Um[kChunk][NC], gam[kChunk], wl[kChunk], bt[kChunk];
-  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-  const int* meta = seq_meta + 4 * s;
-  const int slot = meta[0], first = meta[1], count = meta[2];
-  if (count < min_count) return;
-  const int col0 = blockIdx.z * NC;
-  const int qk_head = h / (H / G);
-  const int v_at = 2 * G * dk + h * dv;
-  float* S = state + static_cast<size_t>(slot) * state_stride + static_cast<size_t>(h) * dk * dv;   // [dv][dk]
-  for (int idx = tid; idx < NC * DK; idx += 256) {
-    const int c = idx / DK, d = idx % DK;
-    Ss[c][d] = (col0 + c < dv && d < dk) ? S[static_cast<size_t>(col0 + c) * dk + d] : 0.f;
-  }
-  const int t = tid / NC, c = tid % NC;        // the element of [32 tokens][NC columns] that this thread computes
-  const int chunks = (count + kChunk - 1) / kChunk;
-  for (int n = 0; n < chunks; ++n) {
-    const int t0 = n * kChunk;
-    const int tn = count - t0 < kChunk ? count - t0 : kChunk;
-    const float* f = scratch + ((static_cast<size_t>(s) * max_chunks + n) * H + h) * kChunkWords;
-    __syncthreads();   // the chunk before has been read to its end
-    for (int idx = tid; idx < kChunk * DK; idx += 256) {
-      const int j = idx / DK, d = idx % DK;
-      const bool ok = j < tn && d < dk;
-      const float* row = qkv + static_cast<size_t>(first + t0 + (ok ? j : 0)) * C;
-      ks[j][d] = ok ? row[(G + qk_head) * dk + d] : 0.f;
-      qs[j][d] = ok ? row[qk_head * dk + d] : 0.f;
-    }
-    for (int idx = tid; idx < kChunk * kChunk; idx += 256) {
-      Tm[idx / kChunk][idx % kChunk] = f[idx];
-      Pm[idx / kChunk][idx % kChunk] = f[kChunk * kChunk + idx];
-    }
-    vs[t][c] = (t < tn && col0 + c < dv) ? qkv[static_cast<size_t>(first + t0 + t) * C + v_at + col0 + c] : 0.f;
-    if (tid < kChunk) {
-      gam[tid] = f[2 * kChunk * kChunk + tid];
-      wl[tid] = f[2 * kChunk * kChunk + kChunk + tid];
-      bt[tid] = f[2 * kChunk * kChunk + 2 * kChunk + tid];
-    }
-    __syncthreads();
-    // S0^T k_t and S0^T q_t for this thread's (t, c)
-    float4 ka = {0.f, 0.f, 0.f, 0.f}, qa = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-    for (int d = 0; d < DK; d += 4) {
-      const float4 k4 = *reinterpret_cast<const float4*>(&ks[t][d]);
-      const float4 q4 = *reinterpret_cast<const float4*>(&qs[t][d]);
-      const float4 s4 = *reinterpret_cast<const float4*>(&Ss[c][d]);
-      ka.x = fmaf(k4.x, s4.x, ka.x); ka.y = fmaf(k4.y, s4.y, ka.y); ka.z = fmaf(k4.z, s4.z, ka.z); ka.w = fmaf(k4.w, s4.w, ka.w);
-      qa.x = fmaf(q4.x, s4.x, qa.x); qa.y = fmaf(q4.y, s4.y, qa.y); qa.z = fmaf(q4.z, s4.z, qa.z); qa.w = fmaf(q4.w, s4.w, qa.w);
-    }
-    const float KS = (ka.x + ka.y) + (ka.z + ka.w), QS = (qa.x + qa.y) + (qa.z + qa.w);
-    Bm[t][c] = bt[t] * (vs[t][c] - gam[t] * KS);
-    __syncthreads();
-    float u = 0.f;
-#pragma unroll 8
-    for (int i = 0; i < kChunk; ++i) u = fmaf(Tm[t][i], Bm[i][c], u);   // (T is 0 above its diagonal)
-    Um[t][c] = u;
-    __syncthreads();
-    float o = gam[t] * QS;
-#pragma unroll 8
-    for (int i = 0; i < kChunk; ++i) o = fmaf(Pm[t][i], Um[i][c], o);   // (P is 0 above its diagonal)
-    if (t < tn && col0 + c < dv)
-      out[static_cast<size_t>(first + t0 + t) * (static_cast<size_t>(H) * dv) + static_cast<size_t>(h) * dv + col0 + c] = o;
-    // the state after the chunk: four neighbouring rows of one column per thread and turn
-    const float g_all = gam[kChunk - 1];
-    for (int piece = tid / NC; piece * 4 < DK; piece += 256 / NC) {
-      const int d = piece * 4;
-      float4 a = *reinterpret_cast<const float4*>(&Ss[c][d]);
-      a.x *= g_all; a.y *= g_all; a.z *= g_all; a.w *= g_all;
-#pragma unroll 8
-      for (int j = 0; j < kChunk; ++j) {
-        const float w = wl[j] * Um[j][c];
-        const float4 k4 = *reinterpret_cast<const float4*>(&ks[j][d]);
-        a.x = fmaf(k4.x, w, a.x); a.y = fmaf(k4.y, w, a.y); a.z = fmaf(k4.z, w, a.z); a.w = fmaf(k4.w, w, a.w);
-      }
-      // (every read of Ss by the products above lies before the last two barriers; this thread alone reads and
-      // writes these four words now)
-      *reinterpret_cast<float4*>(&Ss[c][d]) = a;
-    }
-  }
-  __syncthreads();
-  for (int idx = tid; idx < NC * DK; idx += 256) {
-    const int cc = idx / DK, d = idx % DK;
-    if (col0 + cc < dv && d < dk) S[static_cast<size_t>(col0 + cc) * dk + d] = Ss[cc][d];
   }
 }
 
@@ -478,16 +292,8 @@ extern "C" int sa_delta_prepare(float* qkv, int T, int C, int G, int dk, const v
   return check_launch("delta_prepare");
 }
 
-// How many tokens a request must bring for the chunked kernels to take it (0: they do not take this key size), and
-// the floats of scratch memory that they need for num_seqs requests of at most max_q_len tokens.
-extern "C" int sa_delta_rule_chunk_threshold(int dk) { return (dk <= 128 && dk % 4 == 0) ? 2 * kChunk : 0; }
-extern "C" int64_t sa_delta_rule_scratch_words(int num_seqs, int max_q_len, int H) {
-  return static_cast<int64_t>(num_seqs) * ((max_q_len + kChunk - 1) / kChunk) * H * kChunkWords;
-}
-
 extern "C" int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, const float* gates, int H, float* state,
-                             int64_t state_stride, const int* seq_meta, int num_seqs, int min_q_len, int max_q_len,
-                             float* scratch, int64_t scratch_words, float* out, hipStream_t stream) {
+                             int64_t state_stride, const int* seq_meta, int num_seqs, float* out, hipStream_t stream) {
   if (num_seqs == 0) return 0;
   SA_REQUIRE(num_seqs > 0 && G > 0 && H > 0 && H % G == 0 && dk > 0 && dv > 0 && C >= 2 * G * dk + H * dv,
              "delta_rule: bad sizes S=%d C=%d G=%d H=%d dk=%d dv=%d", num_seqs, C, G, H, dk, dv);
@@ -495,40 +301,15 @@ extern "C" int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, con
   SA_REQUIRE(state_stride >= static_cast<int64_t>(H) * dk * dv, "delta_rule: the state rows are too short");
   SA_REQUIRE(qkv != nullptr && gates != nullptr && state != nullptr && seq_meta != nullptr && out != nullptr,
              "delta_rule: a null pointer");
-  SA_REQUIRE(H <= 65535 && dv <= 65535 * 8 && num_seqs <= 65535, "delta_rule: too many heads, columns or requests");
-  SA_REQUIRE(max_q_len >= 1 && min_q_len >= 0 && min_q_len <= max_q_len, "delta_rule: bad token counts");
-  // requests with many tokens go chunk by chunk (if there is scratch memory for their chunks' factors), the others
-  // token by token
-  int threshold = sa_delta_rule_chunk_threshold(dk);
-  if (threshold == 0 || max_q_len < threshold || scratch == nullptr ||
-      scratch_words < sa_delta_rule_scratch_words(num_seqs, max_q_len, H))
-    threshold = 0x7fffffff;
-  if (max_q_len >= threshold) {
-    const int max_chunks = (max_q_len + kChunk - 1) / kChunk;
-    const dim3 grid1(max_chunks, num_seqs, H), grid2(num_seqs, H, (dv + 7) / 8);
-#define SA_DELTA_CHUNKED(DK)                                                                                          \
-  do {                                                                                                                \
-    delta_chunk_factors_kernel<DK><<<grid1, 256, 0, stream>>>(qkv, C, G, dk, gates, H, seq_meta, threshold, scratch,  \
-                                                              max_chunks);                                           \
-    delta_chunk_scan_kernel<DK><<<grid2, 256, 0, stream>>>(qkv, C, G, dk, dv, H, state, state_stride, seq_meta,        \
-                                                           threshold, scratch, max_chunks, out);                      \
-  } while (0)
-    if (dk <= 32) SA_DELTA_CHUNKED(32);
-    else if (dk <= 64) SA_DELTA_CHUNKED(64);
-    else SA_DELTA_CHUNKED(128);
-#undef SA_DELTA_CHUNKED
-    if (check_launch("delta_rule (chunked)")) return 1;
-    if (min_q_len >= threshold) return 0;   // nobody is left for the token-by-token kernel
-  }
-#define SA_DELTA_RULE(DK, LPC, TT)                                                                                  \
-  delta_rule_kernel<DK, LPC, TT><<<dim3(num_seqs, H, (dv + 256 / LPC - 1) / (256 / LPC)), 256, 0, stream>>>(         \
-      qkv, C, G, dk, dv, gates, H, state, state_stride, seq_meta, out, threshold)
-  // (16 tokens per tile: 32 gave the same time per token of a prompt and cost the decode step a third more)
-  if (dk <= 16) SA_DELTA_RULE(16, 4, 16);
-  else if (dk <= 32) SA_DELTA_RULE(32, 4, 16);
-  else if (dk <= 64) SA_DELTA_RULE(64, 16, 16);
-  else if (dk <= 128) SA_DELTA_RULE(128, 64, 16);
-  else SA_DELTA_RULE(256, 64, 16);
+  SA_REQUIRE(H <= 65535 && dv <= 65535 * 16, "delta_rule: too many heads or columns");
+#define SA_DELTA_RULE(DK, LPC)                                                                                      \
+  delta_rule_kernel<DK, LPC><<<dim3(num_seqs, H, (dv + 256 / LPC - 1) / (256 / LPC)), 256, 0, stream>>>(             \
+      qkv, C, G, dk, dv, gates, H, state, state_stride, seq_meta, out)
+  if (dk <= 16) SA_DELTA_RULE(16, 4);
+  else if (dk <= 32) SA_DELTA_RULE(32, 4);
+  else if (dk <= 64) SA_DELTA_RULE(64, 16);
+  else if (dk <= 128) SA_DELTA_RULE(128, 64);
+  else SA_DELTA_RULE(256, 64);
 #undef SA_DELTA_RULE
   return check_launch("delta_rule");
 }

@@ -66,7 +66,7 @@ _SIGNATURES = {
                                         _L, _P, _P],
     "sa_short_conv_silu": [_P, _I, _L, _P, _I, _I, _P, _L, _P, _I, _I, _P, _I, _I, _P],
     "sa_delta_prepare": [_P, _I, _I, _I, _I, _P, _I, _L, _P, _P, _I, _I, _P, _P],
-    "sa_delta_rule": [_P, _I, _I, _I, _I, _P, _I, _P, _L, _P, _I, _I, _I, _P, _L, _P, _P],
+    "sa_delta_rule": [_P, _I, _I, _I, _I, _P, _I, _P, _L, _P, _I, _P, _P],
     "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _L, _P],
 }
 
@@ -108,10 +108,6 @@ def load() -> ctypes.CDLL:
         lib.sa_gemm_plan.restype = c_int
         lib.sa_philox4x32_10.argtypes = [_P, _P, _P]
         lib.sa_philox4x32_10.restype = None
-        lib.sa_delta_rule_chunk_threshold.argtypes = [_I]
-        lib.sa_delta_rule_chunk_threshold.restype = c_int
-        lib.sa_delta_rule_scratch_words.argtypes = [_I, _I, _I]
-        lib.sa_delta_rule_scratch_words.restype = c_int64
         _lib, _path = lib, path
         return lib
 

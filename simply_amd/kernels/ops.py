@@ -875,8 +875,8 @@ def short_conv_silu(x: torch.Tensor, taps: torch.Tensor, tails: torch.Tensor, se
 def delta_prepare(qkv: torch.Tensor, ab: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, num_heads: int,
                   num_qk_heads: int, key_dim: int) -> torch.Tensor:
     """In place on qkv float32 [T, C] = [G q heads | G k heads | values]: q and k heads to unit length, q also times
-    key_dim ** -0.5.  Returns gates float32 [T, 3 H]: beta = sigmoid(b), then g = exp(-exp(a_log) softplus(a +
-    dt_bias)), then ln g, from ab [T, 2 H] = [a | b]."""
+    key_dim ** -0.5.  Returns gates float32 [T, 2 H]: beta = sigmoid(b), then g = exp(-exp(a_log) softplus(a +
+    dt_bias)), from ab [T, 2 H] = [a | b]."""
     _dev(qkv, ab, a_log, dt_bias)
     T, C = qkv.shape
     H, G = num_heads, num_qk_heads
@@ -888,41 +888,31 @@ def delta_prepare(qkv: torch.Tensor, ab: torch.Tensor, a_log: torch.Tensor, dt_b
     if a_log.numel() != H or dt_bias.numel() != H or a_log.dtype != dt_bias.dtype or not a_log.is_contiguous() \
             or not dt_bias.is_contiguous():
         raise KernelError("delta_prepare: a_log and dt_bias have one entry per head, of one type")
-    gates = torch.empty((T, 3 * H), dtype=torch.float32, device=qkv.device)
+    gates = torch.empty((T, 2 * H), dtype=torch.float32, device=qkv.device)
     _lib.call("sa_delta_prepare", _ptr(qkv), T, C, G, key_dim, _ptr(ab), _code(ab), abs_, _ptr(a_log), _ptr(dt_bias),
               _code(a_log), H, _ptr(gates), _stream())
     return gates
 
 
 def delta_rule(qkv: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int,
-               num_heads: int, num_qk_heads: int, key_dim: int, value_dim: int, *, max_q_len: int | None = None,
-               min_q_len: int = 0) -> torch.Tensor:
+               num_heads: int, num_qk_heads: int, key_dim: int, value_dim: int) -> torch.Tensor:
     """The gated delta rule along each request's tokens, from and into state [slots, >= H * dk * dv] float32 (per
-    slot and head the matrix S [dk, dv], stored column by column: [H][dv][dk]).  qkv float32 [T, C] as `delta_prepare` left it, gates [T, 3 H].  Returns float32 [T, H * dv]."""
+    slot and head the matrix S [dk, dv], stored column by column: [H][dv][dk]).  qkv float32 [T, C] as `delta_prepare` left it, gates [T, 2 H].  Returns float32 [T, H * dv]."""
     _dev(qkv, gates, state, seq_meta)
     T, C = qkv.shape
     H, G, dk, dv = num_heads, num_qk_heads, key_dim, value_dim
     if qkv.dtype != torch.float32 or not qkv.is_contiguous() or C < 2 * G * dk + H * dv:
         raise KernelError("delta_rule: qkv must be contiguous float32 [T, >= 2 G dk + H dv]")
-    if gates.dtype != torch.float32 or tuple(gates.shape) != (T, 3 * H) or not gates.is_contiguous():
-        raise KernelError("delta_rule: gates must be contiguous float32 [T, 3 H]")
+    if gates.dtype != torch.float32 or tuple(gates.shape) != (T, 2 * H) or not gates.is_contiguous():
+        raise KernelError("delta_rule: gates must be contiguous float32 [T, 2 H]")
     if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < H * dk * dv:
         raise KernelError("delta_rule: the state must be float32 [slots, >= H * dk * dv]")
     if seq_meta.dtype != torch.int32 or seq_meta.dim() != 2 or seq_meta.shape[1] != 4 or not seq_meta.is_contiguous() \
             or seq_meta.shape[0] < num_seqs:
         raise KernelError("delta_rule: seq_meta must be int32 [S, 4]")
     out = torch.empty((T, H * dv), dtype=torch.float32, device=qkv.device)
-    # max_q_len, min_q_len: the most and the fewest tokens that a request of the step brings (unknown: all of the
-    # step's, none).  Requests with many tokens are worked through in chunks, whose factors need scratch memory.
-    max_q = T if max_q_len is None else int(max_q_len)
-    min_q = max(0, min(int(min_q_len), max_q))
-    scratch, words = None, 0
-    threshold = int(_lib.load().sa_delta_rule_chunk_threshold(dk))
-    if threshold and max_q >= threshold:
-        words = int(_lib.load().sa_delta_rule_scratch_words(int(num_seqs), max_q, H))
-        scratch = torch.empty(words, dtype=torch.float32, device=qkv.device)
     _lib.call("sa_delta_rule", _ptr(qkv), C, G, dk, dv, _ptr(gates), H, _ptr(state), state.stride(0), _ptr(seq_meta),
-              int(num_seqs), min_q, max_q, _ptr(scratch), words, _ptr(out), _stream())
+              int(num_seqs), _ptr(out), _stream())
     return out
 
 

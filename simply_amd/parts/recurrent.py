@@ -68,8 +68,7 @@ class GatedDelta(Mixer):
         state, tails = cache.state[:, :self.state_words], cache.state[:, self.state_words:]
         qkv = ops.short_conv_silu(proj[:, :C], self.taps, tails, ctx.seq_meta, ctx.num_seqs, ctx.max_q_len)
         gates = ops.delta_prepare(qkv, ab, self.a_log, self.dt_bias, H, G, dk)
-        o = ops.delta_rule(qkv, gates, state, ctx.seq_meta, ctx.num_seqs, H, G, dk, dv, max_q_len=ctx.max_q_len,
-                           min_q_len=min(ctx.q_lens))
+        o = ops.delta_rule(qkv, gates, state, ctx.seq_meta, ctx.num_seqs, H, G, dk, dv)
         z = ops.gated_heads(o, proj[:, C:C + H * dv], H, dv, kind=ops.GATE_SILU, weight=self.norm, eps=self.norm_eps,
                             out_dtype=ctx.dtype)
         return ops.gemm(z, self.o_proj)

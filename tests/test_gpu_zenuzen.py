@@ -42,11 +42,6 @@ def test_recurrence_kernel():
     mech.delta_rule_steps(ops, DEV)
 
 
-def test_recurrence_kernels_in_chunks():
-    mech.delta_rule_steps(ops, DEV, T=400, cuts=(100, 1, 129, 64, 2, 104))
-    mech.delta_rule_long_and_short_together(ops, DEV)
-
-
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_part(dtype):
     mech.attention_part(DEV, dtype)
@@ -78,14 +73,6 @@ def test_cuts_match_plain(tmp_path, name, dtype):
 @pytest.mark.parametrize("name", ["mixed", "only_delta", "aligned"])
 def test_batches_match_alone(tmp_path, name, dtype):
     cases.batches_match_alone(tmp_path, DEV, name, dtype)
-
-
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["mixed", "only_delta"])
-def test_long_portions(tmp_path, name, dtype):
-    """Portions of 64 tokens and more, which the delta rule's kernels work through in chunks of 32, beside cuts that
-    go token by token."""
-    cases.cuts_match_plain(tmp_path, DEV, name, dtype, length=171)
 
 
 def test_pages_of_sixteen_keys(tmp_path):

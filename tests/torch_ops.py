@@ -328,12 +328,10 @@ def delta_prepare(qkv, ab, a_log, dt_bias, num_heads, num_qk_heads, key_dim):
     qkv[:, :2 * G * dk] = qk.reshape(T, -1).to(torch.float32)
     a, b = _f(ab[:, :H]), _f(ab[:, H:2 * H])
     g = torch.exp(-torch.exp(_f(a_log)) * torch.nn.functional.softplus(a + _f(dt_bias), threshold=30.0))
-    lg = -torch.exp(_f(a_log)) * torch.nn.functional.softplus(a + _f(dt_bias), threshold=30.0)
-    return torch.cat([torch.sigmoid(b), g, lg], dim=1).to(torch.float32)
+    return torch.cat([torch.sigmoid(b), g], dim=1).to(torch.float32)
 
 
-def delta_rule(qkv, gates, state, seq_meta, num_seqs, num_heads, num_qk_heads, key_dim, value_dim, *, max_q_len=None,
-               min_q_len=0):
+def delta_rule(qkv, gates, state, seq_meta, num_seqs, num_heads, num_qk_heads, key_dim, value_dim):
     T, C = qkv.shape
     H, G, dk, dv = num_heads, num_qk_heads, key_dim, value_dim
     out = torch.empty((T, H * dv), dtype=torch.float32, device=qkv.device)
