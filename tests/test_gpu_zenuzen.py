@@ -42,6 +42,11 @@ def test_recurrence_kernel():
     mech.delta_rule_steps(ops, DEV)
 
 
+def test_recurrence_kernel_long_portions_and_unequal_requests():
+    mech.delta_rule_steps(ops, DEV, T=400, cuts=(100, 1, 129, 64, 2, 104))
+    mech.delta_rule_long_and_short_together(ops, DEV)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_attention_part(dtype):
     mech.attention_part(DEV, dtype)
@@ -73,6 +78,13 @@ def test_cuts_match_plain(tmp_path, name, dtype):
 @pytest.mark.parametrize("name", ["mixed", "only_delta", "aligned"])
 def test_batches_match_alone(tmp_path, name, dtype):
     cases.batches_match_alone(tmp_path, DEV, name, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["mixed", "only_delta"])
+def test_long_portions(tmp_path, name, dtype):
+    """A prompt of 171 tokens: whole, in long portions, in portions of two tokens and token by token."""
+    cases.cuts_match_plain(tmp_path, DEV, name, dtype, length=171)
 
 
 def test_pages_of_sixteen_keys(tmp_path):

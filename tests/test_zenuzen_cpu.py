@@ -83,6 +83,7 @@ def test_reference_of_the_activated_product():
 
 def test_reference_of_the_recurrence():
     mech.delta_rule_steps(torch_ops, CPU)
+    mech.delta_rule_long_and_short_together(torch_ops, CPU)
 
 
 def test_attention_part(cpu_ops):

@@ -242,9 +242,9 @@ def short_convolution(o, device, dtype):
     assert float(tails[1].abs().max()) == 0.0
 
 
-def delta_rule_steps(o, device):
+def delta_rule_steps(o, device, T=40, cuts=(13, 1, 2, 1, 23)):
     """The recurrence in portions against the plain one; decays close to 0 and close to 1, beta from 0 to 1."""
-    T, H, G, dk, dv = 40, 4, 2, 20, 70
+    H, G, dk, dv = 4, 2, 20, 70
     C = 2 * G * dk + H * dv
     x = rand((T, C), 16)
     ab = rand((T, 2 * H), 17, 3.0)
@@ -259,7 +259,8 @@ def delta_rule_steps(o, device):
                                      x[:, 2 * G * dk:].view(T, H, dv), beta, g)
     state = torch.zeros((3, H * dk * dv + 11), dtype=torch.float32, device=device)
     got, at = [], 0
-    for c in (13, 1, 2, 1, 23):
+    assert sum(cuts) == T
+    for c in cuts:
         part = x[at:at + c].float().contiguous().to(device)
         gates = o.delta_prepare(part, ab[at:at + c].float().contiguous().to(device), a_log.float().to(device),
                                 dt_bias.float().to(device), H, G, dk)
@@ -271,6 +272,45 @@ def delta_rule_steps(o, device):
     close(torch.cat(got), want.reshape(T, H * dv), 3e-5, "outputs")
     close(state[1, :H * dk * dv].view(H, dv, dk).transpose(1, 2), S, 3e-5, "state (stored column by column)")
     assert float(state[0].abs().max()) == 0.0 and float(state[2].abs().max()) == 0.0
+
+
+def delta_rule_long_and_short_together(o, device):
+    """One step with requests of 150, 64, 5 and 1 tokens, each from a state that an earlier step left in its slot:
+    every request's result is what it is alone."""
+    H, G, dk, dv = 3, 1, 32, 12
+    C = 2 * G * dk + H * dv
+    counts = {0: (7, 150), 2: (3, 64), 3: (40, 5), 1: (2, 1)}     # slot -> (tokens of the earlier step, of this one)
+    a_log, dt_bias = torch.tensor([-2.0, 0.0, 1.5], dtype=torch.float64), rand((H,), 60)
+    state = torch.zeros((4, H * dk * dv), dtype=torch.float32, device=device)
+    want, rows, metas, xs, abs_ = {}, 0, [], [], []
+    for slot, (before, now) in counts.items():
+        T = before + now
+        x, ab = rand((T, C), 61 + slot), rand((T, 2 * H), 71 + slot, 2.0)
+        q, k = x[:, :G * dk].view(T, G, dk), x[:, G * dk:2 * G * dk].view(T, G, dk)
+        qn = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * dk ** -0.5
+        kn = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+        g = torch.exp(-torch.exp(a_log) * plain.softplus(ab[:, :H] + dt_bias))
+        out, S = plain.delta_recurrence(qn.repeat_interleave(H, 1), kn.repeat_interleave(H, 1),
+                                        x[:, 2 * G * dk:].view(T, H, dv), torch.sigmoid(ab[:, H:]), g)
+        want[slot] = (out[before:].reshape(now, H * dv), S)
+        # the earlier step, alone
+        part = x[:before].float().contiguous().to(device)
+        gates = o.delta_prepare(part, ab[:before].float().contiguous().to(device), a_log.float().to(device),
+                                dt_bias.float().to(device), H, G, dk)
+        meta = torch.tensor([[slot, 0, before, 0]], dtype=torch.int32, device=device)
+        o.delta_rule(part, gates, state, meta, 1, H, G, dk, dv)
+        metas.append([slot, rows, now, before])
+        xs.append(x[before:])
+        abs_.append(ab[before:])
+        rows += now
+    part = torch.cat(xs).float().contiguous().to(device)
+    gates = o.delta_prepare(part, torch.cat(abs_).float().contiguous().to(device), a_log.float().to(device),
+                            dt_bias.float().to(device), H, G, dk)
+    meta = torch.tensor(metas, dtype=torch.int32, device=device)
+    got = o.delta_rule(part, gates, state, meta, len(metas), H, G, dk, dv).cpu()
+    for slot, first, now, _ in metas:
+        close(got[first:first + now], want[slot][0], 3e-5, f"outputs of slot {slot}")
+        close(state[slot].view(H, dv, dk).transpose(1, 2), want[slot][1], 3e-5, f"state of slot {slot}")
 
 
 # --------------------------------------------------------------------------- the mixers as parts
