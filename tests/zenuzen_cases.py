@@ -4,10 +4,6 @@ it with the kernels replaced by their plain torch references (the `cpu_ops` fixt
 kernels themselves.  Nothing here is read from outside the repository."""
 from __future__ import annotations
 
-import json
-import os
-
-import numpy as np
 import torch
 
 import plain_zenuzen as plain

@@ -5,8 +5,6 @@ takes most of the softmax's sum, a convolution whose taps differ by an order of 
 close to 1."""
 from __future__ import annotations
 
-import math
-
 import torch
 
 import plain_zenuzen as plain
