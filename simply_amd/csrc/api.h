@@ -322,6 +322,15 @@ int sa_short_conv_silu(const void* x, int x_dtype, int64_t x_stride, const void*
 int sa_delta_prepare(float* qkv, int T, int C, int G, int dk, const void* ab, int ab_dtype, int64_t ab_stride,
                      const void* a_log, const void* dt_bias, int vec_dtype, int H, float* gates, hipStream_t stream);
 
+// sa_short_conv_silu (with the tails updated) and sa_delta_prepare in one launch, for steps in which no request brings
+// more than a handful of tokens (sa_delta_inputs_few_takes: decoding): y [T, C] receives the convolved, activated and,
+// for the q and k heads, unit-length channels, gates [T, 2 H] beta and g.
+int sa_delta_inputs_few_takes(int max_q_len, int dk);
+int sa_delta_inputs_few(const void* x, int x_dtype, int64_t x_stride, const void* taps, int taps_dtype, int num_taps,
+                        float* tails, int64_t tail_stride, const int* seq_meta, int num_seqs, int max_q_len, float* y,
+                        int C, int G, int dk, const void* ab, int ab_dtype, int64_t ab_stride, const void* a_log,
+                        const void* dt_bias, int vec_dtype, int H, float* gates, hipStream_t stream);
+
 // The gated delta rule over each request's tokens, from and into state[slot] float32, per head the matrix S [dk, dv]
 // stored column by column ([H][dv][dk]): per head
 // S <- g S; u = beta (v - S^T k); S <- S + k u^T; out = S^T q.  Value head h reads q/k head h / (H / G).

@@ -103,6 +103,96 @@ __global__ __launch_bounds__(kWave) void delta_prepare_kernel(float* __restrict_
   }
 }
 
+// For steps in which every request brings few tokens (decoding): the convolution with silu, the new tails, the
+// unit norms of q and k and the gates in one launch.  A wave per (request, unit); units 0 .. 2 G - 1 are the q and
+// k heads (the wave walks the request's tokens in order with each lane's channels' last inputs in registers, norms
+// each token's head across its lanes, and leaves the tails), the next ones are pieces of 256 value channels, the
+// last one computes beta and g for the request's tokens.  The arithmetic per element is that of the separate
+// kernels, in the same order.
+constexpr int kFewTokens = 16;
+constexpr int kFewChannels = 4;   // channels per lane: key sizes up to 256, value pieces of 256
+template <typename XT>   // the element type of the inputs and of the taps
+__global__ __launch_bounds__(kWave) void delta_inputs_few_kernel(
+    const XT* __restrict__ x, int64_t x_stride, const XT* __restrict__ taps, int n,
+    float* __restrict__ tails, int64_t tail_stride, const int* __restrict__ seq_meta, float* __restrict__ y, int C, int G,
+    int dk, const void* __restrict__ ab, int ab_dtype, int64_t ab_stride, const void* __restrict__ a_log,
+    const void* __restrict__ dt_bias, int vec_dtype, int H, float* __restrict__ gates) {
+  const int* meta = seq_meta + 4 * blockIdx.x;
+  const int slot = meta[0], first = meta[1], count = meta[2];
+  const int unit = blockIdx.y, lane = threadIdx.x;
+  const int value_units = (C - 2 * G * dk + kFewChannels * kWave - 1) / (kFewChannels * kWave);
+  if (unit == 2 * G + value_units) {
+    for (int idx = lane; idx < count * H; idx += kWave) {
+      const int t = first + idx / H, h = idx % H;
+      const float a = load_f(ab, ab_dtype, static_cast<size_t>(t) * ab_stride + h);
+      const float b = load_f(ab, ab_dtype, static_cast<size_t>(t) * ab_stride + H + h);
+      const float z = a + load_f(dt_bias, vec_dtype, h);
+      const float sp = z > 30.f ? z : log1pf(expf(z));
+      gates[static_cast<size_t>(t) * 2 * H + h] = 1.f / (1.f + expf(-b));
+      gates[static_cast<size_t>(t) * 2 * H + H + h] = expf(-expf(load_f(a_log, vec_dtype, h)) * sp);
+    }
+    return;
+  }
+  const bool head = unit < 2 * G;
+  const int c0 = head ? unit * dk : 2 * G * dk + (unit - 2 * G) * kFewChannels * kWave;
+  const int c1 = head ? c0 + dk : (c0 + kFewChannels * kWave < C ? c0 + kFewChannels * kWave : C);
+  float* tail = tails + static_cast<size_t>(slot) * tail_stride;
+  float w[kFewChannels][kMaxTaps], win[kFewChannels][kMaxTaps];
+#pragma unroll
+  for (int k = 0; k < kFewChannels; ++k) {
+    const int c = c0 + lane + k * kWave;
+#pragma unroll
+    for (int i = 0; i < kMaxTaps; ++i) {
+      w[k][i] = (c < c1 && i < n) ? to_float(taps[static_cast<size_t>(c) * n + i]) : 0.f;
+      win[k][i] = (c < c1 && i >= 1 && i < n) ? tail[static_cast<size_t>(i - 1) * C + c] : 0.f;   // the n - 1 before the step
+    }
+  }
+  const float q_scale = unit < G ? 1.f / sqrtf(static_cast<float>(dk)) : 1.f;
+  for (int j = 0; j < count; ++j) {
+    float v[kFewChannels];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < kFewChannels; ++k) {
+      const int c = c0 + lane + k * kWave;
+      v[k] = 0.f;
+      if (c < c1) {
+#pragma unroll
+        for (int i = 0; i + 1 < kMaxTaps; ++i) win[k][i] = win[k][i + 1];
+        const float cur = to_float(x[static_cast<size_t>(first + j) * x_stride + c]);
+#pragma unroll
+        for (int i = 0; i < kMaxTaps; ++i)
+          if (i == n - 1) win[k][i] = cur;
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < kMaxTaps; ++i)
+          if (i < n) acc = fmaf(w[k][i], win[k][i], acc);
+        v[k] = acc / (1.f + expf(-acc));
+        ss = fmaf(v[k], v[k], ss);
+      }
+    }
+    float r = 1.f;
+    if (head) {   // (uniform over the wave)
+      // the sum runs over a lane's channels first and then across the lanes; the separate kernel's runs in the same order
+      ss = wave_sum(ss);
+      r = (1.f / sqrtf(ss + 1e-6f)) * q_scale;
+    }
+#pragma unroll
+    for (int k = 0; k < kFewChannels; ++k) {
+      const int c = c0 + lane + k * kWave;
+      if (c < c1) y[static_cast<size_t>(first + j) * C + c] = head ? v[k] * r : v[k];
+    }
+  }
+  if (count <= 0) return;
+#pragma unroll
+  for (int k = 0; k < kFewChannels; ++k) {
+    const int c = c0 + lane + k * kWave;
+    if (c >= c1) continue;
+#pragma unroll
+    for (int i = 0; i + 1 < kMaxTaps; ++i)
+      if (i + 1 < n) tail[static_cast<size_t>(i) * C + c] = win[k][i + 1];
+  }
+}
+
 // The recurrence.  A workgroup of 256 threads takes 256 / LPC columns of one head's state for one request: LPC lanes
 // (4 or 16, neighbours in a row of 16 lanes) share a column, lane `part` of them holding rows part, part + LPC, ...
 // of it in registers (DK / LPC of them).  The step's q, k and v of kRuleTokens tokens at a time go through LDS.
@@ -290,6 +380,42 @@ extern "C" int sa_delta_prepare(float* qkv, int T, int C, int G, int dk, const v
   delta_prepare_kernel<<<dim3(T, 2 * G + 1), kWave, 0, stream>>>(qkv, C, G, dk, ab, ab_dtype, ab_stride, a_log, dt_bias,
                                                                  vec_dtype, H, gates);
   return check_launch("delta_prepare");
+}
+
+extern "C" int sa_delta_inputs_few_takes(int max_q_len, int dk) {
+  return max_q_len >= 1 && max_q_len <= kFewTokens && dk <= kFewChannels * kWave;
+}
+
+extern "C" int sa_delta_inputs_few(const void* x, int x_dtype, int64_t x_stride, const void* taps, int taps_dtype,
+                                   int num_taps, float* tails, int64_t tail_stride, const int* seq_meta, int num_seqs,
+                                   int max_q_len, float* y, int C, int G, int dk, const void* ab, int ab_dtype,
+                                   int64_t ab_stride, const void* a_log, const void* dt_bias, int vec_dtype, int H,
+                                   float* gates, hipStream_t stream) {
+  if (num_seqs == 0 || max_q_len == 0) return 0;
+  SA_REQUIRE(sa_delta_inputs_few_takes(max_q_len, dk), "delta_inputs_few: at most %d tokens a request and key sizes up to %d",
+             kFewTokens, kFewChannels * kWave);
+  SA_REQUIRE(num_seqs > 0 && num_seqs <= 65535 && C > 0 && G > 0 && dk > 0 && H > 0 && H % G == 0 && C >= 2 * G * dk,
+             "delta_inputs_few: bad sizes S=%d C=%d G=%d dk=%d H=%d", num_seqs, C, G, dk, H);
+  SA_REQUIRE(num_taps >= 1 && num_taps <= kMaxTaps, "delta_inputs_few: 1 to %d taps, got %d", kMaxTaps, num_taps);
+  SA_REQUIRE(x != nullptr && taps != nullptr && (tails != nullptr || num_taps == 1) && seq_meta != nullptr &&
+                 y != nullptr && ab != nullptr && a_log != nullptr && dt_bias != nullptr && gates != nullptr,
+             "delta_inputs_few: a null pointer");
+  SA_REQUIRE(x_stride >= C && ab_stride >= 2 * H && tail_stride >= static_cast<int64_t>(num_taps - 1) * C,
+             "delta_inputs_few: a stride is below what the sizes need");
+  const int value_units = (C - 2 * G * dk + kFewChannels * kWave - 1) / (kFewChannels * kWave);
+  SA_REQUIRE(2 * G + value_units + 1 <= 65535, "delta_inputs_few: too many heads or channels");
+  SA_REQUIRE(x_dtype == taps_dtype && (x_dtype == kF32 || x_dtype == kBF16),
+             "delta_inputs_few: inputs and taps of one element type, float32 or bfloat16");
+  const dim3 grid(num_seqs, 2 * G + value_units + 1);
+  if (x_dtype == kBF16)
+    delta_inputs_few_kernel<bf16><<<grid, kWave, 0, stream>>>(
+        static_cast<const bf16*>(x), x_stride, static_cast<const bf16*>(taps), num_taps, tails, tail_stride, seq_meta, y,
+        C, G, dk, ab, ab_dtype, ab_stride, a_log, dt_bias, vec_dtype, H, gates);
+  else
+    delta_inputs_few_kernel<float><<<grid, kWave, 0, stream>>>(
+        static_cast<const float*>(x), x_stride, static_cast<const float*>(taps), num_taps, tails, tail_stride, seq_meta,
+        y, C, G, dk, ab, ab_dtype, ab_stride, a_log, dt_bias, vec_dtype, H, gates);
+  return check_launch("delta_inputs_few");
 }
 
 extern "C" int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, const float* gates, int H, float* state,

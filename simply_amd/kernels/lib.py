@@ -65,6 +65,8 @@ _SIGNATURES = {
     "sa_paged_attention_prefill_sink": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P,
                                         _L, _P, _P],
     "sa_short_conv_silu": [_P, _I, _L, _P, _I, _I, _P, _L, _P, _I, _I, _P, _I, _I, _P],
+    "sa_delta_inputs_few": [_P, _I, _L, _P, _I, _I, _P, _L, _P, _I, _I, _P, _I, _I, _I, _P, _I, _L, _P, _P, _I, _I, _P, _P],
+    "sa_delta_inputs_few_takes": [_I, _I],
     "sa_delta_prepare": [_P, _I, _I, _I, _I, _P, _I, _L, _P, _P, _I, _I, _P, _P],
     "sa_delta_rule": [_P, _I, _I, _I, _I, _P, _I, _P, _L, _P, _I, _P, _P],
     "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _L, _P],

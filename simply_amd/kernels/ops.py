@@ -894,6 +894,41 @@ def delta_prepare(qkv: torch.Tensor, ab: torch.Tensor, a_log: torch.Tensor, dt_b
     return gates
 
 
+def delta_inputs(x: torch.Tensor, taps: torch.Tensor, tails: torch.Tensor, ab: torch.Tensor, a_log: torch.Tensor,
+                 dt_bias: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int, max_q_len: int, num_heads: int,
+                 num_qk_heads: int, key_dim: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """`short_conv_silu` (the tails updated) followed by `delta_prepare`: returns (qkv float32 [T, C], gates float32
+    [T, 2 H]).  One launch where no request of the step brings more than a handful of tokens (decoding), the two
+    kernels otherwise."""
+    if x.dtype != taps.dtype or not bool(_lib.load().sa_delta_inputs_few_takes(int(max_q_len), int(key_dim))):
+        qkv = short_conv_silu(x, taps, tails, seq_meta, num_seqs, max_q_len)
+        return qkv, delta_prepare(qkv, ab, a_log, dt_bias, num_heads, num_qk_heads, key_dim)
+    _dev(x, taps, tails, ab, a_log, dt_bias, seq_meta)
+    stride = _rows(x, "delta_inputs: x")
+    T, C = x.shape
+    H, G = num_heads, num_qk_heads
+    if taps.dim() != 2 or taps.shape[0] != C or not taps.is_contiguous():
+        raise KernelError(f"delta_inputs: taps {tuple(taps.shape)} for {C} channels")
+    n = taps.shape[1]
+    if tails.dtype != torch.float32 or tails.dim() != 2 or tails.stride(1) != 1 or tails.shape[1] < (n - 1) * C:
+        raise KernelError("delta_inputs: tails must be float32 [slots, >= (taps - 1) * channels]")
+    if seq_meta.dtype != torch.int32 or seq_meta.dim() != 2 or seq_meta.shape[1] != 4 or not seq_meta.is_contiguous() \
+            or seq_meta.shape[0] < num_seqs:
+        raise KernelError("delta_inputs: seq_meta must be int32 [S, 4]")
+    abs_ = _rows(ab, "delta_inputs: ab")
+    if ab.shape[0] != T or ab.shape[1] != 2 * H or C < 2 * G * key_dim:
+        raise KernelError(f"delta_inputs: ab {tuple(ab.shape)} is not [T, 2 H], or too few channels")
+    if a_log.numel() != H or dt_bias.numel() != H or a_log.dtype != dt_bias.dtype or not a_log.is_contiguous() \
+            or not dt_bias.is_contiguous():
+        raise KernelError("delta_inputs: a_log and dt_bias have one entry per head, of one type")
+    qkv = torch.empty((T, C), dtype=torch.float32, device=x.device)
+    gates = torch.empty((T, 2 * H), dtype=torch.float32, device=x.device)
+    _lib.call("sa_delta_inputs_few", _ptr(x), _code(x), stride, _ptr(taps), _code(taps), n, _ptr(tails), tails.stride(0),
+              _ptr(seq_meta), int(num_seqs), int(max_q_len), _ptr(qkv), C, G, int(key_dim), _ptr(ab), _code(ab), abs_,
+              _ptr(a_log), _ptr(dt_bias), _code(a_log), H, _ptr(gates), _stream())
+    return qkv, gates
+
+
 def delta_rule(qkv: torch.Tensor, gates: torch.Tensor, state: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int,
                num_heads: int, num_qk_heads: int, key_dim: int, value_dim: int) -> torch.Tensor:
     """The gated delta rule along each request's tokens, from and into state [slots, >= H * dk * dv] float32 (per

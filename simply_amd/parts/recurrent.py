@@ -66,8 +66,8 @@ class GatedDelta(Mixer):
         proj = ops.gemm(x, self.in_proj)
         ab = ops.gemm(x, self.ab_proj, out_dtype=torch.float32)
         state, tails = cache.state[:, :self.state_words], cache.state[:, self.state_words:]
-        qkv = ops.short_conv_silu(proj[:, :C], self.taps, tails, ctx.seq_meta, ctx.num_seqs, ctx.max_q_len)
-        gates = ops.delta_prepare(qkv, ab, self.a_log, self.dt_bias, H, G, dk)
+        qkv, gates = ops.delta_inputs(proj[:, :C], self.taps, tails, ab, self.a_log, self.dt_bias, ctx.seq_meta,
+                                      ctx.num_seqs, ctx.max_q_len, H, G, dk)
         o = ops.delta_rule(qkv, gates, state, ctx.seq_meta, ctx.num_seqs, H, G, dk, dv)
         z = ops.gated_heads(o, proj[:, C:C + H * dv], H, dv, kind=ops.GATE_SILU, weight=self.norm, eps=self.norm_eps,
                             out_dtype=ctx.dtype)

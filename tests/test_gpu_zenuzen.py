@@ -38,6 +38,11 @@ def test_partial_rotary_into_tiled_pages():
     mech.partial_rotary_norm_and_pages(ops, DEV, torch.bfloat16, page_size=16)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_delta_inputs_of_short_steps(dtype):
+    mech.delta_inputs_of_short_steps(ops, DEV, dtype)
+
+
 def test_recurrence_kernel():
     mech.delta_rule_steps(ops, DEV)
 

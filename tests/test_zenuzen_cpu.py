@@ -81,6 +81,10 @@ def test_reference_of_the_activated_product():
     mech.activated_product(torch_ops, CPU, torch.float32)
 
 
+def test_reference_of_the_delta_inputs():
+    mech.delta_inputs_of_short_steps(torch_ops, CPU, torch.float32)
+
+
 def test_reference_of_the_recurrence():
     mech.delta_rule_steps(torch_ops, CPU)
     mech.delta_rule_long_and_short_together(torch_ops, CPU)

@@ -331,6 +331,11 @@ def delta_prepare(qkv, ab, a_log, dt_bias, num_heads, num_qk_heads, key_dim):
     return torch.cat([torch.sigmoid(b), g], dim=1).to(torch.float32)
 
 
+def delta_inputs(x, taps, tails, ab, a_log, dt_bias, seq_meta, num_seqs, max_q_len, num_heads, num_qk_heads, key_dim):
+    qkv = short_conv_silu(x, taps, tails, seq_meta, num_seqs, max_q_len)
+    return qkv, delta_prepare(qkv, ab, a_log, dt_bias, num_heads, num_qk_heads, key_dim)
+
+
 def delta_rule(qkv, gates, state, seq_meta, num_seqs, num_heads, num_qk_heads, key_dim, value_dim):
     T, C = qkv.shape
     H, G, dk, dv = num_heads, num_qk_heads, key_dim, value_dim

@@ -240,6 +240,47 @@ def short_convolution(o, device, dtype):
     assert float(tails[1].abs().max()) == 0.0
 
 
+def delta_inputs_of_short_steps(o, device, dtype):
+    """Convolution, silu, new tails, unit q and k and the gates as one call, for steps of few tokens a request: two
+    requests over three steps (2 + 1 + 9 tokens and 5 + 7 tokens), against the plain functions on the whole sequences."""
+    H, G, dk, dv, n = 4, 2, 70, 9, 4
+    C = 2 * G * dk + H * dv
+    taps = torch.tensor([1.0, -3.0, 9.0, 0.3], dtype=torch.float64)[None, :] * (1.0 + rand((C, 1), 80, 0.1))
+    a_log, dt_bias = torch.tensor([-2.0, 0.0, 0.5, 1.0], dtype=torch.float64), rand((H,), 81)
+    xs = {0: rand((12, C), 82), 3: rand((12, C), 83)}
+    abs_ = {0: rand((12, 2 * H), 84, 2.0), 3: rand((12, 2 * H), 85, 2.0)}
+    td = taps.to(dtype)
+    want = {}
+    for slot in xs:
+        y = plain.silu(plain.causal_conv(xs[slot].to(dtype).double(), td.double()))
+        q, k = y[:, :G * dk].view(12, G, dk), y[:, G * dk:2 * G * dk].view(12, G, dk)
+        y[:, :G * dk] = (q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * dk ** -0.5).reshape(12, -1)
+        y[:, G * dk:2 * G * dk] = (k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)).reshape(12, -1)
+        ab = abs_[slot].float().double()
+        want[slot] = (y, torch.sigmoid(ab[:, H:]), torch.exp(-torch.exp(a_log) * plain.softplus(ab[:, :H] + dt_bias)))
+    tails = torch.zeros((4, (n - 1) * C), dtype=torch.float32, device=device)
+    done = {0: 0, 3: 0}
+    for step in ([(0, 2), (3, 5)], [(0, 1)], [(3, 7), (0, 9)]):
+        x = torch.cat([xs[s][done[s]:done[s] + c] for s, c in step]).to(dtype).contiguous().to(device)
+        ab = torch.cat([abs_[s][done[s]:done[s] + c] for s, c in step]).float().contiguous().to(device)
+        meta, at = [], 0
+        for s, c in step:
+            meta.append([s, at, c, done[s]])
+            at += c
+        qkv, gates = o.delta_inputs(x, td.to(device), tails, ab, a_log.float().to(device), dt_bias.float().to(device),
+                                    torch.tensor(meta, dtype=torch.int32, device=device), len(step),
+                                    max(c for _, c in step), H, G, dk)
+        for (s, c), (_, first, _, _) in zip(step, meta):
+            y, beta, g = (w[done[s]:done[s] + c] for w in want[s])
+            close(qkv[first:first + c], y, tol_of(dtype), f"slot {s} from {done[s]}")
+            close(gates[first:first + c, :H], beta, 2e-6, "beta")
+            close(gates[first:first + c, H:], g, 2e-5, "decay")
+            done[s] += c
+    for s in xs:
+        close(tails[s].view(n - 1, C), xs[s].to(dtype)[-(n - 1):], 0.0, f"tail of slot {s}")
+    assert float(tails[1].abs().max()) == 0.0 and float(tails[2].abs().max()) == 0.0
+
+
 def delta_rule_steps(o, device, T=40, cuts=(13, 1, 2, 1, 23)):
     """The recurrence in portions against the plain one; decays close to 0 and close to 1, beta from 0 to 1."""
     H, G, dk, dv = 4, 2, 20, 70
