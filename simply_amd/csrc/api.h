@@ -85,7 +85,8 @@ int sa_decode_slots(int B, const int* positions, const int* token_seq, const int
 // C[M, N] = epilogue(A[M, K] . W[N, K]^T).  epilogue 0: none; 1 + 16 * a: act(A.W^T) * (A.W2^T) with the activation
 // a of activations.h (0: tanh-approximated gelu, 1: silu, 2: squared relu), both products rounded to the output
 // type first; 2: cap * tanh(. / cap); 3 + 16 * a: act(A.W^T), the product rounded to the output type first (in
-// the wide kernel's epilogue where that kernel runs without a cut of K, else by a kernel behind the product).  algo 0: the library chooses; 1: the generic 32-bit-ALU kernel; 2: the
+// the epilogue of the few-rows kernel and of the wide kernel where it runs without a cut of K, else by a kernel
+// behind the product).  algo 0: the library chooses; 1: the generic 32-bit-ALU kernel; 2: the
 // few-rows bfloat16 kernel; 3: the tiled bfloat16 MFMA kernel; 4: the wide-tile bfloat16 MFMA kernel for very
 // many rows (2, 3 and 4 refuse what they do not take).
 // packed: W (and W2) are tiled instead of row-major: [ceil(N / 16)][ceil(K / 32)][64][8] bfloat16, block (i, j)

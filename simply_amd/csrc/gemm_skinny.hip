@@ -213,6 +213,9 @@ __global__ __launch_bounds__(1024) void gemm_skinny_kernel(const bf16* __restric
       v = gated_activation(act, to_float(float_to_bf16(v))) * to_float(float_to_bf16(sum[NP - 1]));
     } else if (EPI == 2) {
       v = cap * tanhf(v / cap);
+    } else if (act > 0) {
+      // (without another epilogue, act > 0 asks for the activation act - 1 of the product rounded to bfloat16)
+      v = gated_activation(act - 1, to_float(float_to_bf16(v)));
     }
     store_f(C, c_dtype, static_cast<size_t>(m) * ldc + n, v);
   }

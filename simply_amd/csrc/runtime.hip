@@ -94,6 +94,9 @@ static int gemm_routed(const void* A, int a_dtype, int64_t lda, const void* W, c
   if (kernel == 4)
     return gemm_wide(A, lda, W, C, ldc, M, N, K, epilogue, activated ? activated : act, algo == 4 ? shape % 10000000 : 0,
                      algo == 4 ? shape / 10000000 : 1, workspace, ws_bytes, stream, planes_left);
+  // (the few-rows kernel has the activation in its epilogue too, for bfloat16 results)
+  if (kernel == 2 && activated && c_dtype == kBF16)
+    return gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, activated, cap, packed, shape, stream);
   int rc;
   if (kernel == 2)
     rc = gemm_skinny(A, lda, W, W2, C, c_dtype, ldc, M, N, K, epilogue, act, cap, packed, shape, stream);
