@@ -194,14 +194,14 @@ __global__ __launch_bounds__(kWave) void delta_inputs_few_kernel(
 }
 
 // The recurrence.  A workgroup of 256 threads takes 256 / LPC columns of one head's state for one request: LPC lanes
-// (4 or 16, neighbours in a row of 16 lanes) share a column, lane `part` of them holding rows part, part + LPC, ...
+// (4, 16 or a whole wave of 64) share a column, lane `part` of them holding rows part, part + LPC, ...
 // of it in registers (DK / LPC of them).  The step's q, k and v of kRuleTokens tokens at a time go through LDS.
 // Columns are independent of each other; a column's sums run within a lane over its rows in increasing order, in
 // four partial sums that are added in a fixed order, then across the lanes by data-parallel primitives in a fixed
 // order: nothing depends on how the tokens are cut into steps or on the batch.  The chain of dependent operations
 // per token, and the instructions that one wave issues for it, are what bound a prompt's time (tokens follow one
-// another, and a head's columns are all the waves there are): 16 or 32 lanes per column keep both short where a
-// column has 64 rows or more.
+// another, and a head's columns are all the waves there are): 16 lanes per column, or a wave, keep both short where
+// a column has 64 rows or more.
 constexpr int kRuleTokens = 16;
 template <int LPC>
 __device__ __forceinline__ float lanes_sum(float v) {
