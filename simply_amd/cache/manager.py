@@ -56,7 +56,15 @@ def pages_for_memory(needs, *, page_size: int, num_slots: int, max_seq_len: int,
     more than `num_slots` sequences of `max_seq_len` need, at least one sequence's worth of one page.  `needs` as
     `CacheManager` takes them."""
     per_page_full = per_page_windowed_total = 0
-    for need, cache_from in needs:
+
+    def flat(need):
+        if isinstance(getattr(need, "parts", None), tuple):
+            for n in need.parts:
+                yield from flat(n)
+        else:
+            yield need
+
+    for need, cache_from in ((n, c) for whole, c in needs for n in flat(whole)):
         if cache_from is not None or not callable(getattr(need, "page_tensors", None)):
             continue
         page_bytes = need.bytes_per_token(esize) * page_size
@@ -255,6 +263,8 @@ class CacheView:
     pages: dict = dataclasses.field(default_factory=dict)
     state: torch.Tensor | None = None     # [num_slots, ...] as the need's `slot_tensor` made it
     write: bool = True                    # False: this entry reads the cache of another entry
+    #: for a need made of several parts' needs: one view per part, in the need's order (this view then holds nothing itself)
+    parts: list = dataclasses.field(default_factory=list)
 
     @property
     def k_pages(self) -> torch.Tensor | None:
@@ -292,7 +302,7 @@ class CacheManager:
         #: still to come start there, so a window's pages below what they see can go
         self.issued: dict[Hashable, int] = {}
         self.views: list[CacheView] = []
-        self._group_entries: dict[int, list[int]] = {}
+        self._group_views: dict[int, list[CacheView]] = {}   # per group the views that hold its pages
         self._device_tables: dict[int, torch.Tensor] = {}
         self._stage_host = self._stage_dev = self._stage_done = None  # what `sync_tables` sends its rows through
         by_need: dict[object, CacheGroup] = {}
@@ -303,52 +313,76 @@ class CacheManager:
                 if type(src.need) is not type(need) or src.need != need:
                     raise CacheError(f"schedule entry {i} reads the cache of entry {cache_from}, whose need differs: "
                                      f"{need} vs {src.need}")
-                self.views.append(dataclasses.replace(src, write=False))
+                self.views.append(self._read_only(src))
                 continue
-            if need is None:
-                self.views.append(CacheView(None))
-            elif callable(getattr(need, "page_tensors", None)):
-                # something per token, in pages: layers with equal needs share pool, free list and block table
-                group = by_need.get(need)
-                if group is None:
-                    pages = self.num_pages
-                    window = getattr(need, "window", None)
-                    if window is not None and max_step_tokens is not None:
-                        pages = min(pages, windowed_pool_pages(window, self.page_size, self.num_slots,
-                                                               int(max_step_tokens)))
-                    if group_pages is not None:
-                        pages = int(group_pages(need, pages))
-                    group = CacheGroup(len(self.groups), need, self.page_size, pages, self.num_slots, max_blocks)
-                    by_need[need] = group
-                    self.groups.append(group)
-                    self._group_entries[group.group_id] = []
-                view = CacheView(need, group.group_id)
-                if device is not None:
-                    n = group.pool.num_pages
-                    view.pages = dict(need.page_tensors(n, self.page_size, dtype, device,
-                                                        float("nan") if poison else 0.0))
-                    for name, t in view.pages.items():
-                        if t.dim() < 1 or t.shape[0] != n:
-                            raise CacheError(f"schedule entry {i}: page tensor {name!r} of {need!r} has shape "
-                                             f"{tuple(t.shape)}; its first dimension must be the {n} pages")
-                self._group_entries[group.group_id].append(i)
-                self.views.append(view)
-            elif callable(getattr(need, "slot_tensor", None)):
-                # something of fixed size per request: a row per request slot
-                view = CacheView(need)
-                if device is not None:
-                    view.state = need.slot_tensor(self.num_slots, device)
-                    if view.state.dim() < 1 or view.state.shape[0] != self.num_slots:
-                        raise CacheError(f"schedule entry {i}: the state of {need!r} has shape "
-                                         f"{tuple(view.state.shape)}; its first dimension must be the {self.num_slots} slots")
-                self.views.append(view)
-            else:
-                raise CacheError(f"schedule entry {i}: cache need {need!r} says neither page_tensors(...) (something "
-                                 f"per token) nor slot_tensor(...) (something of fixed size per request)")
+            self.views.append(self._make_view(i, need, by_need, max_blocks, max_step_tokens, group_pages))
         if device is not None:
             for g in self.groups:
                 self._device_tables[g.group_id] = torch.full((self.num_slots, g.max_blocks), -1, dtype=torch.int32,
                                                              device=device)
+
+    def _make_view(self, i: int, need, by_need: dict, max_blocks: int, max_step_tokens, group_pages) -> "CacheView":
+        """The storage of one need of schedule entry i (a need of several parts: a view with one view per part)."""
+        device, dtype, poison = self.device, self.dtype, self.poison
+        if need is None:
+            return CacheView(None)
+        if isinstance(getattr(need, "parts", None), tuple):
+            view = CacheView(need)
+            view.parts = [self._make_view(i, n, by_need, max_blocks, max_step_tokens, group_pages) for n in need.parts]
+            return view
+        if callable(getattr(need, "page_tensors", None)):
+            # something per token, in pages: layers with equal needs share pool, free list and block table
+            group = by_need.get(need)
+            if group is None:
+                pages = self.num_pages
+                window = getattr(need, "window", None)
+                if window is not None and max_step_tokens is not None:
+                    pages = min(pages, windowed_pool_pages(window, self.page_size, self.num_slots,
+                                                           int(max_step_tokens)))
+                if group_pages is not None:
+                    pages = int(group_pages(need, pages))
+                group = CacheGroup(len(self.groups), need, self.page_size, pages, self.num_slots, max_blocks)
+                by_need[need] = group
+                self.groups.append(group)
+                self._group_views[group.group_id] = []
+            view = CacheView(need, group.group_id)
+            if device is not None:
+                n = group.pool.num_pages
+                view.pages = dict(need.page_tensors(n, self.page_size, dtype, device,
+                                                    float("nan") if poison else 0.0))
+                for name, t in view.pages.items():
+                    if t.dim() < 1 or t.shape[0] != n:
+                        raise CacheError(f"schedule entry {i}: page tensor {name!r} of {need!r} has shape "
+                                         f"{tuple(t.shape)}; its first dimension must be the {n} pages")
+            self._group_views[group.group_id].append(view)
+            return view
+        if callable(getattr(need, "slot_tensor", None)):
+            # something of fixed size per request: a row per request slot
+            view = CacheView(need)
+            if device is not None:
+                view.state = need.slot_tensor(self.num_slots, device)
+                if view.state.dim() < 1 or view.state.shape[0] != self.num_slots:
+                    raise CacheError(f"schedule entry {i}: the state of {need!r} has shape "
+                                     f"{tuple(view.state.shape)}; its first dimension must be the {self.num_slots} slots")
+            return view
+        raise CacheError(f"schedule entry {i}: cache need {need!r} says neither page_tensors(...) (something "
+                         f"per token) nor slot_tensor(...) (something of fixed size per request), nor is it made "
+                         f"of parts that do")
+
+    @staticmethod
+    def _read_only(view: "CacheView") -> "CacheView":
+        copy = dataclasses.replace(view, write=False)
+        copy.parts = [CacheManager._read_only(p) for p in view.parts]
+        return copy
+
+    @staticmethod
+    def _leaves(view: "CacheView"):
+        """A view's own storage, or that of its parts."""
+        if view.parts:
+            for p in view.parts:
+                yield from CacheManager._leaves(p)
+        else:
+            yield view
 
     # ------------------------------------------------------------------ requests
     def has_slot(self) -> bool:
@@ -365,9 +399,10 @@ class CacheManager:
         self.issued[rid] = 0
         for g in self.groups:
             g.add(rid, slot)
-        for v in self.views:
-            if v.state is not None and v.write:
-                v.state[slot].zero_()
+        for view in self.views:
+            for v in self._leaves(view):
+                if v.state is not None and v.write:
+                    v.state[slot].zero_()
         return slot
 
     def slot_of(self, rid: Hashable) -> int:
@@ -462,8 +497,8 @@ class CacheManager:
         if not (self.poison and self.device is not None and pages):
             return
         idx = torch.as_tensor(list(pages), dtype=torch.long, device=self.device)
-        for e in self._group_entries[g.group_id]:
-            for t in self.views[e].pages.values():
+        for view in self._group_views[g.group_id]:
+            for t in view.pages.values():
                 if t.is_floating_point():
                     t[idx] = float("nan")
 
@@ -537,4 +572,5 @@ class CacheManager:
     def bytes_per_token(self) -> int:
         """Bytes of cache that one token takes over all schedule entries that keep their own."""
         esize = torch.empty((), dtype=self.dtype).element_size()
-        return sum(v.need.bytes_per_token(esize) for v in self.views if v.group_id is not None and v.write)
+        return sum(v.need.bytes_per_token(esize) for view in self.views for v in self._leaves(view)
+                   if v.group_id is not None and v.write)

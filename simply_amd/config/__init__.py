@@ -12,6 +12,7 @@ from .engine import EngineConfig, parse_dtype
 from .spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
 from .gemma2 import ConfigError, Gemma2Config
 from .zenuzen import ZenuzenConfig
+from .nemidra import NemidraConfig
 
 
 def architecture_name(d: Mapping[str, Any]) -> str:
@@ -24,9 +25,13 @@ def architecture_name(d: Mapping[str, Any]) -> str:
     return str(archs[0])
 
 
-def config_from_dict(d: Mapping[str, Any]):
-    """Typed configuration of the architecture that `d` names."""
-    return ARCHITECTURES.get(architecture_name(d)).from_dict(d)
+def config_from_dict(d: Mapping[str, Any], complete: bool = True):
+    """Typed configuration of the architecture that `d` names.  complete False: sizes that the architecture reads
+    from the tensors' shapes may still be open (`resolve_shapes` closes them)."""
+    cls = ARCHITECTURES.get(architecture_name(d))
+    if not complete and hasattr(cls, "from_dict_open"):
+        return cls.from_dict_open(d)
+    return cls.from_dict(d)
 
 
 def load_config(model_dir: str):
@@ -34,8 +39,14 @@ def load_config(model_dir: str):
     if not os.path.isfile(path):
         raise FileNotFoundError(f"{path}: no config.json in the model folder")
     with open(path) as f:
-        return config_from_dict(json.load(f))
+        config = config_from_dict(json.load(f), complete=False)
+    if hasattr(config, "resolve_shapes"):
+        # sizes that the configuration leaves to the tensors' shapes
+        from ..weights.loader import stored_shapes
+
+        config = config.resolve_shapes(stored_shapes(model_dir))
+    return config
 
 
 __all__ = ["EngineConfig", "parse_dtype", "LayerSpec", "ModelSpec", "PartSpec", "ScheduleEntry",
-           "ConfigError", "Gemma2Config", "ZenuzenConfig", "architecture_name", "config_from_dict", "load_config"]
+           "ConfigError", "Gemma2Config", "ZenuzenConfig", "NemidraConfig", "architecture_name", "config_from_dict", "load_config"]

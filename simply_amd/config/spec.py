@@ -34,15 +34,20 @@ class LayerSpec:
     mixer: PartSpec
     feed_forward: "PartSpec | None"
     norms: Mapping[str, PartSpec] = dataclasses.field(default_factory=dict)
+    #: parts that update the residual stream themselves at the block's end (registry STREAM_PARTS), in their order
+    extras: "tuple[PartSpec, ...]" = ()
 
 
 @dataclasses.dataclass(frozen=True)
 class ScheduleEntry:
-    """Run layer `layer`.  `cache_from` names an earlier schedule entry (by its index
+    """Run layer `layer` (a layer may be named by several entries: each has a cache or state of its own).  `cache_from` names an earlier schedule entry (by its index
     in the schedule) whose cache this entry reads instead of keeping its own."""
 
     layer: int
     cache_from: int | None = None
+    #: the embedding's output of this step is added to the residual stream before this entry runs (a pass of a loop
+    #: over layers that is given the input again)
+    add_embedding: bool = False
 
 
 @dataclasses.dataclass(frozen=True)
@@ -61,6 +66,9 @@ class ModelSpec:
     #: tensor names that a model folder may hold beside the expected ones, each with the expected tensor whose
     #: copy it must be (a tied head stored once more under its own name): checked for equality, then left unread
     copies: Mapping[str, str] = dataclasses.field(default_factory=dict)
+    #: tensor names that a model folder may hold and that the model does not read (norms around a feed-forward that
+    #: a layer does not have)
+    ignorable: tuple[str, ...] = ()
 
     def validate(self) -> None:
         n = len(self.layers)

@@ -8,7 +8,7 @@
 
 namespace sa {
 
-enum Activation : int { kActGeluTanh = 0, kActSilu = 1, kActSquaredRelu = 2, kNumActivations = 3 };
+enum Activation : int { kActGeluTanh = 0, kActSilu = 1, kActSquaredRelu = 2, kActGeluErf = 3, kNumActivations = 4 };
 
 // kEpilogueActivated: C = act(A.W^T), the product rounded to the output type first (a feed-forward without a gate)
 constexpr int kEpilogueNone = 0, kEpilogueGated = 1, kEpilogueSoftCap = 2, kEpilogueActivated = 3;
@@ -26,12 +26,15 @@ __device__ inline float gelu_tanh_fast(float x) {
 // x * sigmoid(x) with the hardware's exponential and reciprocal; exact at both ends (exp(-x) = inf gives x * 0).
 __device__ inline float silu_fast(float x) { return x * __builtin_amdgcn_rcpf(1.f + __expf(-x)); }
 __device__ inline float squared_relu(float x) { return x > 0.f ? x * x : 0.f; }
+// x * Phi(x) with the library's error function: the exact GELU.
+__device__ inline float gelu_erf(float x) { return 0.5f * x * (1.f + erff(x * 0.7071067811865476f)); }
 
 // For the bfloat16 kernels.
 __device__ inline float gated_activation(int act, float x) {
   switch (act) {
     case kActSilu: return silu_fast(x);
     case kActSquaredRelu: return squared_relu(x);
+    case kActGeluErf: return gelu_erf(x);
     default: return gelu_tanh_fast(x);
   }
 }
@@ -41,6 +44,7 @@ __device__ inline float gated_activation_exact(int act, float x) {
   switch (act) {
     case kActSilu: return x / (1.f + expf(-x));
     case kActSquaredRelu: return squared_relu(x);
+    case kActGeluErf: return gelu_erf(x);
     default: return 0.5f * x * (1.f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
   }
 }

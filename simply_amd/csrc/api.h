@@ -350,4 +350,61 @@ int sa_paged_attention_prefill_sink(const void* q, int64_t q_stride, const void*
                                     int unit_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,
                                     int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
                                     void* workspace, int64_t workspace_bytes, const float* sinks, hipStream_t stream);
+// ---- token tables
+// out[t, :] = table[token] + pair[(previous * mul_prev + token * mul_cur) mod buckets] + pos[position]; a request's
+// first token takes the pair table's row `buckets`; the token before a step's first one is last[slot], which is then
+// set to the step's last token of the request.  pair, pos: null to leave them out.
+int sa_embed_sum(const int* tokens, const int* positions, const int* seq_meta, int num_seqs, int max_q_len,
+                 const void* table, int table_dtype, int V, const void* pair, int pair_dtype, int64_t buckets,
+                 int64_t mul_prev, int64_t mul_cur, int* last, int64_t last_stride, const void* pos, int pos_dtype,
+                 int max_positions, float* out, int D, hipStream_t stream);
+// z[t, j] = act(z[t, j]) * table[tokens[t], col0 + j], in place.
+int sa_token_gate(void* z, int dtype, int64_t stride, const int* tokens, const void* table, int table_dtype,
+                  int64_t table_stride, int col0, int T, int N, int act, hipStream_t stream);
+// x[t, n] += b[n], in place.
+int sa_bias_add(void* x, int dtype, int64_t stride, const void* b, int b_dtype, int T, int N, hipStream_t stream);
+// out = a x + b y.
+int sa_weighted_sum(const void* x, int64_t x_stride, float a, const void* y, int64_t y_stride, float b, int dtype,
+                    void* out, int64_t out_stride, int T, int N, hipStream_t stream);
+
+// ---- matrix states that decay (linear_state.hip)
+// decay[t, c] = sigmoid(z)^(1 / tau), z = w2[c, :] . u[t, :] + b[c].
+int sa_gla_decay(const void* u, int u_dtype, int64_t u_stride, const void* w2, int w_dtype, const void* b, int b_dtype,
+                 float tau, int T, int R, int C, float* decay, hipStream_t stream);
+// raw [T, 2 H] (input gates, forget gates), bias [2 H] or null -> gates [T, 3 H]: decay, input factor, exp(-m), with
+// the running maximum m of every (slot, head) read from and left in m_state[slot * state_stride + h].
+int sa_exp_gates(const float* raw, int64_t raw_stride, const void* bias, int bias_dtype, float cap, int H,
+                 float* m_state, int64_t state_stride, const int* seq_meta, int num_seqs, float* gates,
+                 hipStream_t stream);
+// S <- diag(a) S + c k v^T, out = S^T (q * q_mult) along every request's tokens; q, k, v are columns q_at, k_at, v_at
+// of proj's rows.  scalar: gates [T, >= 2 H] hold a and c per head; else gates [T, H dk] hold a per key channel and
+// c = 1.  ones: the state has a column dv whose value is always 1.  state [slot][H][dv + ones][dk]; out [T, H (dv + ones)].
+int sa_linear_state(const void* proj, int dtype, int64_t proj_stride, int q_at, int k_at, int v_at, float q_mult,
+                    const float* gates, int64_t gates_stride, int scalar, int H, int dk, int dv, int ones, float* state,
+                    int64_t state_stride, const int* seq_meta, int num_seqs, float* out, hipStream_t stream);
+// x [T, H, size + 1] -> out[t, h, :] = unit_rms(x[t, h, :size] / (max(|x[t, h, size]|, floor[t, h]) + 1e-6)) * w[h, :]
+// * sigmoid(g[t, h, :]).
+int sa_normalized_readout(const float* x, const float* floor, int64_t floor_stride, const void* g, int g_dtype,
+                          int64_t g_stride, const void* w, int w_dtype, float eps, void* out, int out_dtype,
+                          int64_t out_stride, int T, int H, int size, hipStream_t stream);
+
+// ---- routed experts (routed.hip)
+// softmax over E logits, the top largest: experts [T, top], weights [T, top] = score * scale.
+int sa_route(const float* logits, int64_t stride, int T, int E, int top, float scale, int* experts, float* weights,
+             hipStream_t stream);
+// The most tiles of 16 rows of one expert that P pairs over E experts make.
+int sa_expert_tiles_max(int P, int E);
+// sorted [P]: the pairs by expert; plan [1 + 2 * sa_expert_tiles_max(P, E)]: the tiles.
+int sa_expert_sort(const int* experts, int P, int E, int* sorted, int* plan, int plan_words, hipStream_t stream);
+// w2 given: out[row] = act(a . w1[e]^T) * (a . w2[e]^T) in a's type; else out[row] = a . w1[e]^T in 32-bit.  a's row is
+// the pair's token (a_by_token) or its place in the sorted order; out's row the pair (out_by_pair) or that place.
+// bfloat16 weights are tiled [E][ceil(N / 16)][ceil(K / 32)][64][8], 32-bit ones row-major [E][N][K].
+int sa_expert_product(const void* a, int dtype, int64_t a_stride, int a_by_token, int top, const void* w1, const void* w2,
+                      int N, int K, const int* sorted, const int* plan, int P, int E, int act, void* out,
+                      int64_t out_stride, int out_by_pair, hipStream_t stream);
+// out[t] = sum_k weights[t, k] y[t * top + k] + sigmoid(gate[t]) * shared[t]  (shared null: none; gate null: 1).
+int sa_expert_combine(const float* y, const float* weights, int top, const void* shared, int shared_dtype,
+                      int64_t shared_stride, const float* gate, int64_t gate_stride, void* out, int out_dtype,
+                      int64_t out_stride, int T, int D, hipStream_t stream);
+
 }

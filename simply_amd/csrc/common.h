@@ -83,6 +83,28 @@ __device__ inline float wave_max(float v) {
   return wave_combine(v, [](float a, float b) { return fmaxf(a, b); });
 }
 
+// The sum of a value over groups of LPC neighbouring lanes (4, 16, 32 or 64), in every lane of the group, in a fixed order.
+template <int LPC>
+__device__ __forceinline__ float lanes_sum(float v) {
+  v += lane_exchange<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+  v += lane_exchange<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  if (LPC >= 16) {
+    v += lane_exchange<0x141>(v);  // row_half_mirror
+    v += lane_exchange<0x140>(v);  // row_mirror
+  }
+  if (LPC >= 32) {   // two rows of 16 lanes: gfx950's row swap brings the neighbouring row's sum
+    const unsigned u = __float_as_uint(v);
+    const auto rows = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    v = __uint_as_float(rows[0]) + __uint_as_float(rows[1]);
+  }
+  if (LPC == 64) {   // and the other half of the wave
+    const unsigned u = __float_as_uint(v);
+    const auto halves = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    v = __uint_as_float(halves[0]) + __uint_as_float(halves[1]);
+  }
+  return v;
+}
+
 // Sum over a block of up to 1024 threads; every thread gets the result.  The
 // order of additions depends only on the block size, never on the data.
 __device__ inline float block_sum(float v, float* scratch /* >= 16 floats */) {

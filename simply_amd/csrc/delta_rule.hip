@@ -203,27 +203,6 @@ __global__ __launch_bounds__(kWave) void delta_inputs_few_kernel(
 // another, and a head's columns are all the waves there are): 16 lanes per column, or a wave, keep both short where
 // a column has 64 rows or more.
 constexpr int kRuleTokens = 16;
-template <int LPC>
-__device__ __forceinline__ float lanes_sum(float v) {
-  v += lane_exchange<0xB1>(v);   // quad_perm [1, 0, 3, 2]
-  v += lane_exchange<0x4E>(v);   // quad_perm [2, 3, 0, 1]
-  if (LPC >= 16) {
-    v += lane_exchange<0x141>(v);  // row_half_mirror
-    v += lane_exchange<0x140>(v);  // row_mirror
-  }
-  if (LPC >= 32) {   // two rows of 16 lanes: gfx950's row swap brings the neighbouring row's sum
-    const unsigned u = __float_as_uint(v);
-    const auto rows = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-    v = __uint_as_float(rows[0]) + __uint_as_float(rows[1]);
-  }
-  if (LPC == 64) {   // and the other half of the wave
-    const unsigned u = __float_as_uint(v);
-    const auto halves = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    v = __uint_as_float(halves[0]) + __uint_as_float(halves[1]);
-  }
-  return v;
-}
-
 template <int DK, int LPC>
 __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict__ qkv, int C, int G, int dk, int dv,
                                                          const float* __restrict__ gates, int H,

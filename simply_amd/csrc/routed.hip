@@ -1,0 +1,276 @@
+// A feed-forward of routed experts over a ragged batch of tokens.
+//
+//   route_kernel          softmax of the router's logits, the `top` largest scores and their experts
+//   sort_kernel           the (token, choice) pairs in the order of their experts, cut into tiles of rows of one expert
+//   expert_gate_up_kernel h = act(Wg[e] x) * (Wu[e] x) for every pair, rows in the sorted order
+//   expert_down_kernel    y = Wd[e] h, one row per pair (in the pairs' own order)
+//   combine_kernel        out[t] = sum_k weight[t, k] y[t, k] + sigmoid(s[t]) * shared[t]
+//
+// Nothing comes back to the host between them: the tiles are found on the device, and the grid of the expert
+// kernels is sized for the most tiles that the pairs can make.  Every pair's row is computed by itself, with sums
+// in an order that depends on the sizes alone, so a token's result does not depend on the batch.  Scores are
+// 32-bit; the products are bfloat16 on the matrix cores (32-bit accumulation) or 32-bit on the vector unit.
+#include "api.h"
+#include "common.h"
+
+namespace sa {
+
+constexpr int kRouteSlots = 8;    // experts per lane: up to 512 experts
+constexpr int kTileRows = 16;     // rows of a tile: one MFMA operand
+
+// A wave per token.  scores = softmax(logits); `top` times the largest score that is left (of equal ones the lowest
+// index); weight = score * scale.
+__global__ __launch_bounds__(kWave) void route_kernel(const float* __restrict__ logits, int64_t stride, int E, int top,
+                                                      float scale, int* __restrict__ experts,
+                                                      float* __restrict__ weights) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  float z[kRouteSlots];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < kRouteSlots; ++i) {
+    const int e = lane + i * kWave;
+    z[i] = e < E ? logits[static_cast<size_t>(t) * stride + e] : -INFINITY;
+    mx = fmaxf(mx, z[i]);
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < kRouteSlots; ++i) {
+    z[i] = (lane + i * kWave) < E ? expf(z[i] - mx) : -1.f;   // (a score is never negative: -1 marks what is taken or absent)
+    sum += z[i] > 0.f ? z[i] : 0.f;
+  }
+  sum = wave_sum(sum);
+  for (int r = 0; r < top; ++r) {
+    float best = -1.f;
+#pragma unroll
+    for (int i = 0; i < kRouteSlots; ++i) best = fmaxf(best, z[i]);
+    best = wave_max(best);
+    float mine = 1e9f;
+#pragma unroll
+    for (int i = kRouteSlots - 1; i >= 0; --i)
+      if (z[i] == best) mine = static_cast<float>(lane + i * kWave);
+    const float first = -wave_max(-mine);
+    const int e = static_cast<int>(first);
+#pragma unroll
+    for (int i = 0; i < kRouteSlots; ++i)
+      if (lane + i * kWave == e) z[i] = -1.f;
+    if (lane == 0) {
+      experts[static_cast<size_t>(t) * top + r] = e;
+      weights[static_cast<size_t>(t) * top + r] = best / sum * scale;
+    }
+  }
+}
+
+// One workgroup.  plan: [0] number of tiles; [1 .. 1 + 2 * max_tiles): per tile its expert and its first row in the
+// sorted order with the number of its rows packed as first * 32 + rows.  sorted [P]: pair indices by expert.
+__global__ __launch_bounds__(1024) void sort_kernel(const int* __restrict__ experts, int P, int E,
+                                                    int* __restrict__ sorted, int* __restrict__ plan, int max_tiles) {
+  extern __shared__ int lds[];   // counts [E], offsets [E + 1], tile offsets [E + 1], cursors [E]
+  int* counts = lds;
+  int* offsets = lds + E;
+  int* tiles = offsets + E + 1;
+  int* cursor = tiles + E + 1;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) atomicAdd(&counts[experts[p]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, nt = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = at;
+      tiles[e] = nt;
+      at += counts[e];
+      nt += (counts[e] + kTileRows - 1) / kTileRows;
+    }
+    offsets[E] = at;
+    tiles[E] = nt;
+    plan[0] = nt < max_tiles ? nt : max_tiles;
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    cursor[e] = 0;
+    for (int i = 0; tiles[e] + i < tiles[e + 1]; ++i) {
+      const int n = tiles[e] + i;
+      if (n >= max_tiles) break;
+      const int rows = counts[e] - i * kTileRows < kTileRows ? counts[e] - i * kTileRows : kTileRows;
+      plan[1 + 2 * n] = e;
+      plan[2 + 2 * n] = (offsets[e] + i * kTileRows) * 32 + rows;
+    }
+  }
+  __syncthreads();
+  // (the order of an expert's rows among themselves is whatever the atomics give: every row is computed by itself)
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = experts[p];
+    sorted[offsets[e] + atomicAdd(&cursor[e], 1)] = p;
+  }
+}
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+__device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+
+// h[row, f] = act(x[token] . Wg[e, f]) * (x[token] . Wu[e, f]); GATED false: y[pair, n] = h[row] . Wd[e, n].
+// A workgroup of four waves takes one tile of rows and 64 columns (a wave 16 of them).
+// bfloat16: the weights are tiled ([E][N / 16][K / 32][64][8], see the product kernels), a wave's operands are one
+// 16-byte load a lane; 32-bit: row-major weights [E][N][K], a lane per (row, column) of the tile in turn.
+template <typename T, bool GATED>
+__global__ __launch_bounds__(256) void expert_product_kernel(
+    const T* __restrict__ a, int64_t a_stride, int a_by_token, int top, const T* __restrict__ w1, const T* __restrict__ w2,
+    int N, int K, const int* __restrict__ sorted, const int* __restrict__ plan, int act, void* __restrict__ out,
+    int64_t out_stride, int out_by_pair) {
+  const int tile = blockIdx.x;
+  if (tile >= plan[0]) return;
+  const int e = plan[1 + 2 * tile], packed = plan[2 + 2 * tile];
+  const int row0 = packed / 32, rows = packed % 32;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int n0 = (blockIdx.y * 4 + wave) * 16;
+  if (n0 >= N) return;
+  if constexpr (sizeof(T) == 2) {
+    const int Nt = (N + 15) / 16, Kt = (K + 31) / 32;
+    const int r = lane % 16, kq = lane / 16;
+    const int rr = r < rows ? r : rows - 1;
+    const int pair = sorted[row0 + rr];
+    const T* arow = a + static_cast<size_t>(a_by_token ? pair / top : row0 + rr) * a_stride;
+    const size_t wbase = (static_cast<size_t>(e) * Nt + n0 / 16) * Kt;
+    const bf16* g = reinterpret_cast<const bf16*>(w1) + wbase * 512 + lane * 8;
+    const bf16* u = GATED ? reinterpret_cast<const bf16*>(w2) + wbase * 512 + lane * 8 : nullptr;
+    floatx4 accg = {0.f, 0.f, 0.f, 0.f}, accu = {0.f, 0.f, 0.f, 0.f};
+    for (int kt = 0; kt < Kt; ++kt) {
+      const int k = kt * 32 + kq * 8;
+      bf16x8 av;
+      if (k + 8 <= K) {
+        av = load8(reinterpret_cast<const bf16*>(arow) + k);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) av[i] = k + i < K ? __builtin_bit_cast(__bf16, reinterpret_cast<const bf16*>(arow)[k + i]) : static_cast<__bf16>(0.f);
+      }
+      // the weights' rows are the product's columns: C^T = W . A^T, a lane holds four rows (columns of the
+      // output) of one token
+      accg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load8(g + static_cast<size_t>(kt) * 512), av, accg, 0, 0, 0);
+      if constexpr (GATED)
+        accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load8(u + static_cast<size_t>(kt) * 512), av, accu, 0, 0, 0);
+    }
+    // lane: token r = lane % 16, output columns n0 + kq * 4 + i
+    if (r < rows) {
+      const size_t orow = static_cast<size_t>(out_by_pair ? pair : row0 + r) * out_stride;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + kq * 4 + i;
+        if (n >= N) continue;
+        if constexpr (GATED) {
+          const float v = gated_activation(act, to_float(float_to_bf16(accg[i]))) * to_float(float_to_bf16(accu[i]));
+          static_cast<bf16*>(out)[orow + n] = float_to_bf16(v);
+        } else {
+          static_cast<float*>(out)[orow + n] = accg[i];
+        }
+      }
+    }
+  } else {
+    // 32-bit: 16 columns x up to 16 rows of the tile over the wave's 64 lanes, four rows a lane
+    const int c = lane % 16, n = n0 + c;
+    for (int r = lane / 16; r < rows; r += 4) {
+      const int pair = sorted[row0 + r];
+      const T* arow = a + static_cast<size_t>(a_by_token ? pair / top : row0 + r) * a_stride;
+      if (n >= N) continue;
+      const T* g = w1 + (static_cast<size_t>(e) * N + n) * K;
+      float sg = 0.f, su = 0.f;
+      for (int k = 0; k < K; ++k) sg = fmaf(to_float(arow[k]), to_float(g[k]), sg);
+      const size_t orow = static_cast<size_t>(out_by_pair ? pair : row0 + r) * out_stride;
+      if constexpr (GATED) {
+        const T* u = w2 + (static_cast<size_t>(e) * N + n) * K;
+        for (int k = 0; k < K; ++k) su = fmaf(to_float(arow[k]), to_float(u[k]), su);
+        static_cast<float*>(out)[orow + n] = gated_activation_exact(act, sg) * su;
+      } else {
+        static_cast<float*>(out)[orow + n] = sg;
+      }
+    }
+  }
+}
+
+// out[t, d] = sum_k weights[t, k] * y[t * top + k, d] (in the order of k) + sigmoid(gate[t]) * shared[t, d].
+__global__ void combine_kernel(const float* __restrict__ y, const float* __restrict__ weights, int top,
+                               const void* __restrict__ shared, int shared_dtype, int64_t shared_stride,
+                               const float* __restrict__ gate, int64_t gate_stride, void* __restrict__ out, int out_dtype,
+                               int64_t out_stride, int D) {
+  const int t = blockIdx.y, d = blockIdx.x * blockDim.x + threadIdx.x;
+  if (d >= D) return;
+  float v = 0.f;
+  for (int k = 0; k < top; ++k)
+    v = fmaf(weights[static_cast<size_t>(t) * top + k], y[(static_cast<size_t>(t) * top + k) * D + d], v);
+  if (shared != nullptr) {
+    const float s = load_f(shared, shared_dtype, static_cast<size_t>(t) * shared_stride + d);
+    v += gate != nullptr ? s / (1.f + expf(-gate[static_cast<size_t>(t) * gate_stride])) : s;
+  }
+  store_f(out, out_dtype, static_cast<size_t>(t) * out_stride + d, v);
+}
+
+}  // namespace sa
+
+using namespace sa;
+
+extern "C" int sa_route(const float* logits, int64_t stride, int T, int E, int top, float scale, int* experts,
+                        float* weights, hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(T > 0 && E > 0 && E <= kRouteSlots * kWave && top > 0 && top <= E && stride >= E,
+             "route: bad sizes T=%d E=%d top=%d (at most %d experts)", T, E, top, kRouteSlots * kWave);
+  SA_REQUIRE(logits != nullptr && experts != nullptr && weights != nullptr, "route: a null pointer");
+  route_kernel<<<T, kWave, 0, stream>>>(logits, stride, E, top, scale, experts, weights);
+  return check_launch("route");
+}
+
+extern "C" int sa_expert_tiles_max(int P, int E) { return (P + kTileRows - 1) / kTileRows + (E < P ? E : P); }
+
+extern "C" int sa_expert_sort(const int* experts, int P, int E, int* sorted, int* plan, int plan_words,
+                              hipStream_t stream) {
+  if (P == 0) return 0;
+  const int max_tiles = sa_expert_tiles_max(P, E);
+  SA_REQUIRE(P > 0 && E > 0 && E <= 4096 && P < (1 << 26), "expert_sort: bad sizes P=%d E=%d", P, E);
+  SA_REQUIRE(plan_words >= 1 + 2 * max_tiles, "expert_sort: the plan needs %d words", 1 + 2 * max_tiles);
+  SA_REQUIRE(experts != nullptr && sorted != nullptr && plan != nullptr, "expert_sort: a null pointer");
+  const int threads = P >= 1024 ? 1024 : ((P + kWave - 1) / kWave) * kWave;
+  sort_kernel<<<1, threads, (4 * E + 2) * sizeof(int), stream>>>(experts, P, E, sorted, plan, max_tiles);
+  return check_launch("expert_sort");
+}
+
+extern "C" int sa_expert_product(const void* a, int dtype, int64_t a_stride, int a_by_token, int top, const void* w1,
+                                 const void* w2, int N, int K, const int* sorted, const int* plan, int P, int E, int act,
+                                 void* out, int64_t out_stride, int out_by_pair, hipStream_t stream) {
+  if (P == 0) return 0;
+  SA_REQUIRE(P > 0 && E > 0 && N > 0 && K > 0 && top > 0 && a_stride >= K && out_stride >= N,
+             "expert_product: bad sizes P=%d E=%d N=%d K=%d", P, E, N, K);
+  SA_REQUIRE(a != nullptr && w1 != nullptr && sorted != nullptr && plan != nullptr && out != nullptr,
+             "expert_product: a null pointer");
+  SA_REQUIRE(act >= 0 && act < kNumActivations, "expert_product: unknown activation %d", act);
+  SA_REQUIRE(dtype == kF32 || dtype == kBF16, "expert_product: unknown dtype %d", dtype);
+  SA_REQUIRE(dtype == kF32 || (a_stride % 8 == 0), "expert_product: bfloat16 rows must be 16-byte aligned");
+  const dim3 grid(sa_expert_tiles_max(P, E), (N + 63) / 64);
+  SA_REQUIRE(grid.y <= 65535, "expert_product: too many columns");
+  const bool gated = w2 != nullptr;
+#define SA_EXPERT(T, G)                                                                                                \
+  expert_product_kernel<T, G><<<grid, 256, 0, stream>>>(static_cast<const T*>(a), a_stride, a_by_token, top,            \
+                                                         static_cast<const T*>(w1), static_cast<const T*>(w2), N, K,   \
+                                                         sorted, plan, act, out, out_stride, out_by_pair)
+  if (dtype == kBF16) {
+    if (gated) SA_EXPERT(bf16, true);
+    else SA_EXPERT(bf16, false);
+  } else {
+    if (gated) SA_EXPERT(float, true);
+    else SA_EXPERT(float, false);
+  }
+#undef SA_EXPERT
+  return check_launch("expert_product");
+}
+
+extern "C" int sa_expert_combine(const float* y, const float* weights, int top, const void* shared, int shared_dtype,
+                                 int64_t shared_stride, const float* gate, int64_t gate_stride, void* out, int out_dtype,
+                                 int64_t out_stride, int T, int D, hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(T > 0 && T <= 65535 && D > 0 && top > 0 && out_stride >= D, "expert_combine: bad sizes T=%d D=%d top=%d", T, D,
+             top);
+  SA_REQUIRE(y != nullptr && weights != nullptr && out != nullptr, "expert_combine: a null pointer");
+  SA_REQUIRE(shared == nullptr || shared_stride >= D, "expert_combine: the shared rows are too short");
+  combine_kernel<<<dim3((D + 255) / 256, T), 256, 0, stream>>>(y, weights, top, shared, shared_dtype, shared_stride, gate,
+                                                               gate_stride, out, out_dtype, out_stride, D);
+  return check_launch("expert_combine");
+}

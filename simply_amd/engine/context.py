@@ -39,6 +39,8 @@ class StepContext:
     #: what a layer leaves for later layers of the same step, by a name that the two agree on (the values of the
     #: step's tokens that a later attention layer mixes into its own): tensors over the step's tokens, gone with the step
     carry: dict = dataclasses.field(default_factory=dict)
+    #: the step's token ids, int32 [T] on the device (for parts that read tables by token)
+    tokens: torch.Tensor | None = None
     #: set for a step whose launches are recorded and replayed for later steps: the most keys that any step that
     #: replays them may have (kernels size their plans by `max_kv_len`, which is then this bound)
     kv_bound: int = 0

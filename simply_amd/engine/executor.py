@@ -395,7 +395,7 @@ class Executor:
         ctx = StepContext(dtype=self.dtype, num_tokens=T, positions=dev[cap:cap + T], token_seq=dev[2 * cap:2 * cap + T],
                           seq_meta=dev[self._meta_at:self._meta_at + 4 * len(entries)].view(len(entries), 4),
                           groups=groups, request_ids=ctx_ids, seq_slots=ctx_slots, seq_starts=ctx_starts, q_lens=ctx_q,
-                          cu_q_lens=cu, to_device=self._to_device)
+                          cu_q_lens=cu, to_device=self._to_device, tokens=dev[:T])
         self._extra_used = 0
         logit_rows = dev[3 * cap:3 * cap + R] if R else None
         return T, R, ctx, logit_rows, [(rid, start, len(e.tokens)) for (rid, start, _), e in zip(wants, entries)], \

@@ -69,6 +69,18 @@ _SIGNATURES = {
     "sa_delta_inputs_few_takes": [_I, _I],
     "sa_delta_prepare": [_P, _I, _I, _I, _I, _P, _I, _L, _P, _P, _I, _I, _P, _P],
     "sa_delta_rule": [_P, _I, _I, _I, _I, _P, _I, _P, _L, _P, _I, _P, _P],
+    "sa_embed_sum": [_P, _P, _P, _I, _I, _P, _I, _I, _P, _I, _L, _L, _L, _P, _L, _P, _I, _I, _P, _I, _P],
+    "sa_token_gate": [_P, _I, _L, _P, _P, _I, _L, _I, _I, _I, _I, _P],
+    "sa_bias_add": [_P, _I, _L, _P, _I, _I, _I, _P],
+    "sa_weighted_sum": [_P, _L, _F, _P, _L, _F, _I, _P, _L, _I, _I, _P],
+    "sa_gla_decay": [_P, _I, _L, _P, _I, _P, _I, _F, _I, _I, _I, _P, _P],
+    "sa_exp_gates": [_P, _L, _P, _I, _F, _I, _P, _L, _P, _I, _P, _P],
+    "sa_linear_state": [_P, _I, _L, _I, _I, _I, _F, _P, _L, _I, _I, _I, _I, _I, _P, _L, _P, _I, _P, _P],
+    "sa_normalized_readout": [_P, _P, _L, _P, _I, _L, _P, _I, _F, _P, _I, _L, _I, _I, _I, _P],
+    "sa_route": [_P, _L, _I, _I, _I, _F, _P, _P, _P],
+    "sa_expert_sort": [_P, _I, _I, _P, _P, _I, _P],
+    "sa_expert_product": [_P, _I, _L, _I, _I, _P, _P, _I, _I, _P, _P, _I, _I, _I, _P, _L, _I, _P],
+    "sa_expert_combine": [_P, _P, _I, _P, _I, _L, _P, _L, _P, _I, _L, _I, _I, _P],
     "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _L, _P],
 }
 
@@ -108,6 +120,8 @@ def load() -> ctypes.CDLL:
             fn.restype = c_int
         lib.sa_gemm_plan.argtypes = [_I, _I, _I, _I, _I, _L, _P]
         lib.sa_gemm_plan.restype = c_int
+        lib.sa_expert_tiles_max.argtypes = [_I, _I]
+        lib.sa_expert_tiles_max.restype = c_int
         lib.sa_philox4x32_10.argtypes = [_P, _P, _P]
         lib.sa_philox4x32_10.restype = None
         _lib, _path = lib, path

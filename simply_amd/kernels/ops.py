@@ -375,11 +375,11 @@ def decode_slots(positions: torch.Tensor, token_seq: torch.Tensor, block_table: 
 
 EPILOGUE_NONE, EPILOGUE_GATED, EPILOGUE_SOFT_CAP, EPILOGUE_ACTIVATED = 0, 1, 2, 3
 #: activations of the gated epilogue (simply_amd/csrc/activations.h); the epilogue argument is 1 + 16 * activation
-ACT_GELU_TANH, ACT_SILU, ACT_SQUARED_RELU = 0, 1, 2
+ACT_GELU_TANH, ACT_SILU, ACT_SQUARED_RELU, ACT_GELU_ERF = 0, 1, 2, 3
 
 
 def _gated(activation: int) -> int:
-    if activation not in (ACT_GELU_TANH, ACT_SILU, ACT_SQUARED_RELU):
+    if activation not in (ACT_GELU_TANH, ACT_SILU, ACT_SQUARED_RELU, ACT_GELU_ERF):
         raise KernelError(f"unknown activation code {activation!r}")
     return EPILOGUE_GATED + 16 * activation
 
@@ -1046,3 +1046,210 @@ def philox4x32_10(counter: tuple[int, int, int, int], key: tuple[int, int]) -> t
     o = (ctypes.c_uint32 * 4)()
     _lib.load().sa_philox4x32_10(c, k, o)
     return tuple(int(v) for v in o)
+
+
+# --------------------------------------------------------------------------- token tables, biases, sums of two mixers
+
+def _seq_meta(seq_meta: torch.Tensor, num_seqs: int, what: str) -> None:
+    if seq_meta.dtype != torch.int32 or seq_meta.dim() != 2 or seq_meta.shape[1] != 4 or not seq_meta.is_contiguous() \
+            or seq_meta.shape[0] < num_seqs:
+        raise KernelError(f"{what}: seq_meta must be int32 [S, 4]")
+
+
+def embed_sum(tokens: torch.Tensor, positions: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int, max_q_len: int,
+              table: torch.Tensor, *, pair: torch.Tensor | None = None, mul_prev: int = 0, mul_cur: int = 0,
+              last: torch.Tensor | None = None, pos: torch.Tensor | None = None) -> torch.Tensor:
+    """float32 [T, D]: table[token] + pair[(previous * mul_prev + token * mul_cur) mod buckets] + pos[position].  pair
+    [buckets + 1, D]: its last row is a request's first token's; `last` int32 [slots, 1] holds every slot's last
+    token and is brought up to date.  pair, pos: None to leave them out."""
+    _dev(tokens, positions, seq_meta, table, pair, last, pos)
+    T = tokens.shape[0]
+    _i32(tokens, "embed_sum: tokens")
+    _i32(positions, "embed_sum: positions", T)
+    _seq_meta(seq_meta, num_seqs, "embed_sum")
+    V, D = table.shape
+    for name, t in (("table", table), ("pair", pair), ("pos", pos)):
+        if t is not None and (t.dim() != 2 or t.shape[1] != D or not t.is_contiguous()):
+            raise KernelError(f"embed_sum: {name} must be a contiguous table of rows of {D}")
+    if pair is not None:
+        if last is None or last.dtype != torch.int32 or last.dim() != 2 or last.stride(1) != 1:
+            raise KernelError("embed_sum: a table of pairs needs the slots' last tokens, int32 [slots, >= 1]")
+        if pair.shape[0] < 2:
+            raise KernelError("embed_sum: the table of pairs has at least one bucket and the first token's row")
+    out = torch.empty((T, D), dtype=torch.float32, device=tokens.device)
+    _lib.call("sa_embed_sum", _ptr(tokens), _ptr(positions), _ptr(seq_meta), int(num_seqs), int(max_q_len), _ptr(table),
+              _code(table), V, _ptr(pair), _code(pair) if pair is not None else 0,
+              (pair.shape[0] - 1) if pair is not None else 0, int(mul_prev), int(mul_cur), _ptr(last),
+              last.stride(0) if last is not None else 0, _ptr(pos), _code(pos) if pos is not None else 0,
+              pos.shape[0] if pos is not None else 0, _ptr(out), D, _stream())
+    return out
+
+
+def token_gate_(z: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, col0: int, activation: int) -> torch.Tensor:
+    """z[t, j] = act(z[t, j]) * table[tokens[t], col0 + j], in place."""
+    _dev(z, tokens, table)
+    T, N = z.shape
+    _i32(tokens, "token_gate_: tokens", T)
+    if table.dim() != 2 or table.stride(1) != 1 or col0 < 0 or col0 + N > table.shape[1]:
+        raise KernelError(f"token_gate_: columns {col0}..{col0 + N} of a table {tuple(table.shape)}")
+    _lib.call("sa_token_gate", _ptr(z), _code(z), _rows(z, "token_gate_: z"), _ptr(tokens), _ptr(table), _code(table),
+              table.stride(0), int(col0), T, N, int(activation), _stream())
+    return z
+
+
+def bias_add_(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """x[t, :] += bias, in place (the sum in 32-bit)."""
+    _dev(x, bias)
+    T, N = x.shape
+    if bias.numel() != N or not bias.is_contiguous():
+        raise KernelError(f"bias_add_: {bias.numel()} biases for rows of {N}")
+    _lib.call("sa_bias_add", _ptr(x), _code(x), _rows(x, "bias_add_: x"), _ptr(bias), _code(bias), T, N, _stream())
+    return x
+
+
+def weighted_sum(x: torch.Tensor, a: float, y: torch.Tensor, b: float, out: torch.Tensor | None = None) -> torch.Tensor:
+    """a * x + b * y."""
+    _dev(x, y, out)
+    if x.shape != y.shape or x.dtype != y.dtype:
+        raise KernelError("weighted_sum: the two terms differ in shape or type")
+    if out is None:
+        out = torch.empty_like(x, memory_format=torch.contiguous_format)
+    if out.shape != x.shape or out.dtype != x.dtype:
+        raise KernelError("weighted_sum: bad output")
+    T, N = x.shape
+    _lib.call("sa_weighted_sum", _ptr(x), _rows(x, "weighted_sum: x"), float(a), _ptr(y), _rows(y, "weighted_sum: y"),
+              float(b), _code(x), _ptr(out), _rows(out, "weighted_sum: out"), T, N, _stream())
+    return out
+
+
+# --------------------------------------------------------------------------- matrix states that decay
+
+def gla_decay(u: torch.Tensor, w2: torch.Tensor, bias: torch.Tensor | None, tau: float) -> torch.Tensor:
+    """float32 [T, C]: sigmoid(u . w2^T + bias)^(1 / tau).  u [T, R] (rows of a projection), w2 [C, R] row-major."""
+    _dev(u, w2, bias)
+    T, R = u.shape
+    if w2.dim() != 2 or w2.shape[1] != R or not w2.is_contiguous():
+        raise KernelError(f"gla_decay: the second factor {tuple(w2.shape)} does not go with rows of {R}")
+    C = w2.shape[0]
+    if bias is not None and (bias.numel() != C or not bias.is_contiguous()):
+        raise KernelError("gla_decay: one bias per channel")
+    out = torch.empty((T, C), dtype=torch.float32, device=u.device)
+    _lib.call("sa_gla_decay", _ptr(u), _code(u), _rows(u, "gla_decay: u"), _ptr(w2), _code(w2), _ptr(bias),
+              _code(bias) if bias is not None else 0, float(tau), T, R, C, _ptr(out), _stream())
+    return out
+
+
+def exp_gates(raw: torch.Tensor, bias: torch.Tensor | None, cap: float, num_heads: int, m_state: torch.Tensor,
+              seq_meta: torch.Tensor, num_seqs: int) -> torch.Tensor:
+    """The gates of a matrix memory with exponential gates.  raw float32 [T, 2 H] (input gates' projections, then forget
+    gates'), bias [2 H] or None, m_state float32 [slots, H] (a view with a row stride): every slot's running maximum,
+    brought up to date.  Returns float32 [T, 3 H]: decay, input factor, exp(-maximum)."""
+    _dev(raw, bias, m_state, seq_meta)
+    T, H = raw.shape[0], int(num_heads)
+    if raw.dtype != torch.float32 or raw.shape[1] != 2 * H:
+        raise KernelError("exp_gates: raw must be float32 [T, 2 H]")
+    if bias is not None and (bias.numel() != 2 * H or not bias.is_contiguous()):
+        raise KernelError("exp_gates: one bias per gate and head")
+    if m_state.dtype != torch.float32 or m_state.dim() != 2 or m_state.shape[1] != H or m_state.stride(1) != 1:
+        raise KernelError("exp_gates: the maxima must be float32 [slots, H]")
+    _seq_meta(seq_meta, num_seqs, "exp_gates")
+    out = torch.empty((T, 3 * H), dtype=torch.float32, device=raw.device)
+    _lib.call("sa_exp_gates", _ptr(raw), _rows(raw, "exp_gates: raw"), _ptr(bias), _code(bias) if bias is not None else 0,
+              float(cap), H, _ptr(m_state), m_state.stride(0), _ptr(seq_meta), int(num_seqs), _ptr(out), _stream())
+    return out
+
+
+def linear_state(proj: torch.Tensor, q_at: int, k_at: int, v_at: int, q_mult: float, gates: torch.Tensor, scalar: bool,
+                 num_heads: int, key_dim: int, value_dim: int, ones: bool, state: torch.Tensor, seq_meta: torch.Tensor,
+                 num_seqs: int) -> torch.Tensor:
+    """S <- diag(a) S + c k v^T, o = S^T (q * q_mult) along each request's tokens, from and into state float32 [slots,
+    >= H * dk * (dv + ones)] (per head [dv + ones][dk]).  q, k, v: columns q_at, k_at, v_at of proj's rows, H heads
+    each.  scalar: gates float32 [T, >= 2 H] hold a and c per head; else [T, H * dk] hold a per key channel, c = 1.
+    ones: one more column whose value is always 1 (a normalizer).  Returns float32 [T, H * (dv + ones)]."""
+    _dev(proj, gates, state, seq_meta)
+    T = proj.shape[0]
+    H, dk, dv, CT = int(num_heads), int(key_dim), int(value_dim), int(value_dim) + int(bool(ones))
+    if gates.dtype != torch.float32 or gates.shape[0] != T:
+        raise KernelError("linear_state: gates must be float32 with one row per token")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < H * dk * CT:
+        raise KernelError("linear_state: the state must be float32 [slots, >= H * dk * (dv + ones)]")
+    _seq_meta(seq_meta, num_seqs, "linear_state")
+    out = torch.empty((T, H * CT), dtype=torch.float32, device=proj.device)
+    _lib.call("sa_linear_state", _ptr(proj), _code(proj), _rows(proj, "linear_state: proj"), int(q_at), int(k_at), int(v_at),
+              float(q_mult), _ptr(gates), _rows(gates, "linear_state: gates"), int(bool(scalar)), H, dk, dv,
+              int(bool(ones)), _ptr(state), state.stride(0), _ptr(seq_meta), int(num_seqs), _ptr(out), _stream())
+    return out
+
+
+def normalized_readout(x: torch.Tensor, floor: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float,
+                       num_heads: int, size: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """x float32 [T, H * (size + 1)] (per head its `size` outputs and the normalizer's product with the query), floor
+    float32 [T, H] (a view): out[t, h] = unit_rms(x / (max(|n . q|, floor) + 1e-6)) * weight[h] * sigmoid(gate[t, h])."""
+    _dev(x, floor, gate, weight)
+    T, H, size = x.shape[0], int(num_heads), int(size)
+    if x.dtype != torch.float32 or not x.is_contiguous() or x.shape[1] != H * (size + 1):
+        raise KernelError("normalized_readout: x must be contiguous float32 [T, H * (size + 1)]")
+    if floor.dtype != torch.float32 or tuple(floor.shape) != (T, H):
+        raise KernelError("normalized_readout: floor must be float32 [T, H]")
+    if tuple(gate.shape) != (T, H * size) or weight.numel() != H * size or not weight.is_contiguous():
+        raise KernelError("normalized_readout: gate [T, H * size] and weight [H * size] expected")
+    out = torch.empty((T, H * size), dtype=out_dtype, device=x.device)
+    _lib.call("sa_normalized_readout", _ptr(x), _ptr(floor), _rows(floor, "normalized_readout: floor"), _ptr(gate),
+              _code(gate), _rows(gate, "normalized_readout: gate"), _ptr(weight), _code(weight), float(eps), _ptr(out),
+              _code(out), H * size, T, H, size, _stream())
+    return out
+
+
+# --------------------------------------------------------------------------- routed experts
+
+def route(logits: torch.Tensor, top: int, scale: float) -> tuple[torch.Tensor, torch.Tensor]:
+    """softmax over the experts' logits (float32 [T, E]); returns (experts int32 [T, top], weights float32 [T, top] =
+    score * scale) of the `top` largest scores, largest first."""
+    _dev(logits)
+    T, E = logits.shape
+    if logits.dtype != torch.float32:
+        raise KernelError("route: the router's logits are float32")
+    experts = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    _lib.call("sa_route", _ptr(logits), _rows(logits, "route: logits"), T, E, int(top), float(scale), _ptr(experts),
+              _ptr(weights), _stream())
+    return experts, weights
+
+
+def routed_experts(x: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor, gate_w, up_w, down_w, activation: int,
+                   *, shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None,
+                   out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """sum_k weights[t, k] * down[e](act(gate[e] x) * (up[e] x)) with e = experts[t, k], plus sigmoid(shared_gate[t]) *
+    shared[t] (shared None: nothing; shared_gate None: shared as it is).  gate_w, up_w, down_w: `packing.ExpertStack`s
+    (every expert's matrix, tiled if bfloat16).  x [T, D] in the weights' type; shared_gate float32 [T, 1]."""
+    _dev(x, experts, weights, gate_w.data, up_w.data, down_w.data, shared, shared_gate)
+    T, D = x.shape
+    top, E, F = experts.shape[1], gate_w.experts, gate_w.rows
+    if (up_w.experts, up_w.rows, up_w.cols) != (E, F, D) or gate_w.cols != D or (down_w.experts, down_w.rows, down_w.cols) != (E, D, F):
+        raise KernelError("routed_experts: the experts' matrices do not go together")
+    if x.dtype != gate_w.data.dtype or gate_w.tiled != (x.dtype == torch.bfloat16):
+        raise KernelError("routed_experts: bfloat16 rows go with tiled weights, float32 rows with row-major ones")
+    if experts.dtype != torch.int32 or not experts.is_contiguous() or tuple(weights.shape) != (T, top) \
+            or weights.dtype != torch.float32 or not weights.is_contiguous():
+        raise KernelError("routed_experts: experts int32 [T, top] and weights float32 [T, top] expected")
+    P = T * top
+    dev = x.device
+    max_tiles = _lib.load().sa_expert_tiles_max(P, E)
+    sorted_ = torch.empty(P, dtype=torch.int32, device=dev)
+    plan = torch.empty(1 + 2 * max_tiles, dtype=torch.int32, device=dev)
+    _lib.call("sa_expert_sort", _ptr(experts), P, E, _ptr(sorted_), _ptr(plan), plan.numel(), _stream())
+    h = torch.empty((P, F), dtype=x.dtype, device=dev)
+    _lib.call("sa_expert_product", _ptr(x), _code(x), _rows(x, "routed_experts: x"), 1, top, _ptr(gate_w.data),
+              _ptr(up_w.data), F, D, _ptr(sorted_), _ptr(plan), P, E, int(activation), _ptr(h), F, 0, _stream())
+    y = torch.empty((P, D), dtype=torch.float32, device=dev)
+    _lib.call("sa_expert_product", _ptr(h), _code(h), F, 0, top, _ptr(down_w.data), None, D, F, _ptr(sorted_), _ptr(plan), P,
+              E, 0, _ptr(y), D, 1, _stream())
+    out = torch.empty((T, D), dtype=out_dtype or x.dtype, device=dev)
+    if shared is not None and tuple(shared.shape) != (T, D):
+        raise KernelError("routed_experts: the shared expert's rows do not match")
+    if shared_gate is not None and (shared_gate.dtype != torch.float32 or shared_gate.shape[0] != T):
+        raise KernelError("routed_experts: the shared expert's gate is float32 [T, 1]")
+    _lib.call("sa_expert_combine", _ptr(y), _ptr(weights), top, _ptr(shared), _code(shared) if shared is not None else 0,
+              _rows(shared, "routed_experts: shared") if shared is not None else 0, _ptr(shared_gate),
+              shared_gate.stride(0) if shared_gate is not None else 0, _ptr(out), _code(out), D, T, D, _stream())
+    return out

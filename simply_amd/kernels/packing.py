@@ -87,6 +87,28 @@ def unpack_tiles(tw: TiledWeight) -> torch.Tensor:
     return full[:tw.rows, :tw.cols].contiguous()
 
 
+@dataclasses.dataclass
+class ExpertStack:
+    """The matrices [N, K] of a set of experts as one tensor: bfloat16 on the GPU tiled like a product weight, expert by
+    expert ([E, ceil(N / 16), ceil(K / 32), 64, 8]); anything else row-major [E, N, K]."""
+
+    data: torch.Tensor
+    experts: int
+    rows: int
+    cols: int
+    tiled: bool
+
+
+def stack_experts(ws) -> ExpertStack:
+    ws = list(ws)
+    N, K = ws[0].shape
+    if any(tuple(w.shape) != (N, K) or w.dtype != ws[0].dtype for w in ws):
+        raise ValueError("stack_experts: the experts' matrices differ in shape or type")
+    if ws[0].dtype == torch.bfloat16 and ws[0].is_cuda:
+        return ExpertStack(torch.stack([pack_tiles(w.contiguous()).data for w in ws]).contiguous(), len(ws), N, K, True)
+    return ExpertStack(torch.stack([w.contiguous() for w in ws]).contiguous(), len(ws), N, K, False)
+
+
 def clear_cache() -> None:
     _cache.clear()
 

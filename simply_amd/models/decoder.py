@@ -15,7 +15,7 @@ from .. import parts as _parts  # noqa: F401  (registers the built-in parts)
 from ..config.spec import LayerSpec, ModelSpec, PartSpec
 from ..kernels import ops
 from ..parts.base import Block, ParamSpec, Part, PendingNorm
-from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS
+from ..registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, STREAM_PARTS
 from ..weights import binding
 
 
@@ -23,6 +23,9 @@ def _build_layer(spec: LayerSpec) -> Block:
     mixer = MIXERS.build(spec.mixer.kind, **spec.mixer.params)
     ffn = None if spec.feed_forward is None else FEED_FORWARDS.build(spec.feed_forward.kind, **spec.feed_forward.params)
     norms = {name: NORMS.build(ns.kind, **ns.params) for name, ns in spec.norms.items()}
+    if spec.extras:
+        extras = tuple(STREAM_PARTS.build(es.kind, **es.params) for es in spec.extras)
+        return BLOCKS.build(spec.block.kind, mixer, ffn, norms, extras=extras, **spec.block.params)
     return BLOCKS.build(spec.block.kind, mixer, ffn, norms, **spec.block.params)
 
 
@@ -45,6 +48,8 @@ class DecoderModel:
                 out.append((block.feed_forward, ls.feed_forward))
             for name, ns in ls.norms.items():
                 out.append((block.norms[name], ns))
+            for part, es in zip(getattr(block, "extras", ()), ls.extras):
+                out.append((part, es))
         out.append((self.final_norm, self.spec.final_norm))
         out.append((self.head, self.spec.head))
         return out
@@ -97,22 +102,45 @@ class DecoderModel:
 
     # ------------------------------------------------------------------ cache
     def cache_needs(self):
-        """For each schedule entry: (need of its mixer or None, cache_from)."""
-        return [(self.layers[e.layer].mixer.cache_need(), e.cache_from) for e in self.spec.schedule]
+        """For each schedule entry: (need of its mixer or None, cache_from); then, if the embedding keeps something
+        per request, one more entry for it (its view is the one behind the schedule's)."""
+        needs = [(self.layers[e.layer].mixer.cache_need(), e.cache_from) for e in self.spec.schedule]
+        own = getattr(self.embedding, "cache_need", None)
+        if own is not None and own() is not None:
+            needs.append((own(), None))
+        return needs
 
     # ------------------------------------------------------------------ forward
     def forward(self, tokens: torch.Tensor, ctx, cache_views, logit_rows: torch.Tensor | None,
-                logits_out: torch.Tensor | None = None) -> torch.Tensor | None:
+                logits_out: torch.Tensor | None = None, after_layer=None) -> torch.Tensor | None:
         """Runs this step's tokens through the schedule.  Returns float32 logits [R, V] at the rows of
         the step that `logit_rows` (int32 [R]) names (in `logits_out` if that is given), or None if it is None or
-        empty."""
-        h = self.embedding.forward(tokens)
+        empty.  `after_layer(i, h)`, if given, is shown the residual stream behind every schedule entry (tests,
+        inspection: every pending sum is then done at once)."""
         schedule = self.spec.schedule
+        if getattr(self.embedding, "needs_context", False):
+            own = len(cache_views) > len(schedule)
+            h = self.embedding.forward(tokens, ctx, cache_views[len(schedule)] if own else None)
+        else:
+            h = self.embedding.forward(tokens)
+        # a pass of a loop that is given the input again adds the embedding's output to the stream
+        again = h.clone() if any(e.add_embedding for e in schedule) else None
         normed = None
         for i, entry in enumerate(schedule):
             block = self.layers[entry.layer]
-            nxt = self.layers[schedule[i + 1].layer].first_norm() if i + 1 < len(schedule) else None
+            if entry.add_embedding:
+                if isinstance(normed, PendingNorm):
+                    h = normed.settle()
+                ops.residual_add_norm(again, h)
+                normed = None
+            nxt = None
+            if i + 1 < len(schedule) and not schedule[i + 1].add_embedding:
+                nxt = self.layers[schedule[i + 1].layer].first_norm()
             h, normed = block.forward(h, ctx, cache_views[i], normed, nxt)
+            if after_layer is not None:
+                if isinstance(normed, PendingNorm):
+                    h = normed.settle()
+                after_layer(i, h)
         if logit_rows is None or logit_rows.numel() == 0:
             return None
         if isinstance(normed, PendingNorm):

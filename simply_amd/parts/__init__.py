@@ -1,6 +1,7 @@
 """Parts that blocks are put together from; importing this package registers the built-in ones."""
-from .base import Block, FeedForward, Mixer, Norm, PagedKVNeed, ParamSpec, Part, PositionEncoding, StateNeed
-from . import attention, block, embedding, ffn, norm, recurrent, rope  # noqa: F401  (registration)
+from .base import (Block, CompositeNeed, FeedForward, Mixer, Norm, PagedKVNeed, ParamSpec, Part, PositionEncoding,
+                   StateNeed, StreamPart)
+from . import attention, block, embedding, ffn, linear_state, norm, parallel, recurrent, rope, side  # noqa: F401  (registration)
 
-__all__ = ["Block", "FeedForward", "Mixer", "Norm", "PagedKVNeed", "ParamSpec", "Part", "PositionEncoding",
-           "StateNeed"]
+__all__ = ["Block", "CompositeNeed", "FeedForward", "Mixer", "Norm", "PagedKVNeed", "ParamSpec", "Part",
+           "PositionEncoding", "StateNeed", "StreamPart"]

@@ -109,21 +109,22 @@ class SinkAttention(Mixer):
       value_mix          'source': the values of the step's tokens are left for later layers under `value_mix_key`;
                          'mix': v <- (1 - vmix) v + vmix (those values), before the cache is written;
       output_gate        the heads are multiplied by sigmoid(gate projection of the mixer's input) before the output
-                         projection.
+                         projection;
+      bias               q, k, v and the output projection have biases.
 
     q, k, v and the gate are one product."""
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, scale: float,
                  sinks: bool = False, qk_norm_eps: float | None = None, output_gate: bool = False,
                  value_mix: str | None = None, value_mix_key: str = "values", window: int | None = None,
-                 position_encoding: PartSpec | None = None):
+                 position_encoding: PartSpec | None = None, bias: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"sink_attention: {num_heads} heads do not split over {num_kv_heads} kv heads")
         if value_mix not in (None, "source", "mix"):
             raise ValueError(f"sink_attention: value_mix is None, 'source' or 'mix', not {value_mix!r}")
         self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
         self.key_dim, self.value_dim, self.scale = int(key_dim), int(value_dim), float(scale)
-        self.sinks, self.output_gate = bool(sinks), bool(output_gate)
+        self.sinks, self.output_gate, self.bias = bool(sinks), bool(output_gate), bool(bias)
         self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.value_mix, self.value_mix_key = value_mix, str(value_mix_key)
         self.window = int(window) if window else None
@@ -131,7 +132,7 @@ class SinkAttention(Mixer):
                                   if position_encoding is not None else None)
         if self.position_encoding is not None and not hasattr(self.position_encoding, "frequencies"):
             raise ValueError("sink_attention: the position encoding must give frequencies() (partial_rope)")
-        self.in_proj = self.o_proj = self.sink = self.vmix = None
+        self.in_proj = self.o_proj = self.sink = self.vmix = self.in_bias = self.o_bias = None
 
     def param_specs(self):
         D, H, K, dk, dv = self.hidden_size, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
@@ -141,6 +142,11 @@ class SinkAttention(Mixer):
             specs["gate_proj"] = ParamSpec((H * dv, D))
         if self.sinks:
             specs["sink"] = ParamSpec((H,), role="vector", init="norm")
+        if self.bias:
+            specs.update(q_bias=ParamSpec((H * dk,), role="vector", init="norm"),
+                         k_bias=ParamSpec((K * dk,), role="vector", init="norm"),
+                         v_bias=ParamSpec((K * dv,), role="vector", init="norm"),
+                         o_bias=ParamSpec((D,), role="vector", init="norm"))
         if self.value_mix is not None:   # (a source stores the factor too and leaves it unused)
             specs["vmix"] = ParamSpec((), role="vector", init="norm")
         return specs
@@ -151,6 +157,12 @@ class SinkAttention(Mixer):
             rows.append(tensors["gate_proj"])
         self.in_proj = as_product_weight(torch.cat(rows, dim=0).contiguous())
         self.o_proj = as_product_weight(tensors["o_proj"])
+        if self.bias:
+            parts = [tensors["q_bias"], tensors["k_bias"], tensors["v_bias"]]
+            if self.output_gate:
+                parts.append(torch.zeros_like(tensors["q_bias"][:1]).expand(self.num_heads * self.value_dim))
+            self.in_bias = torch.cat([p.to(parts[0].dtype) for p in parts]).contiguous()
+            self.o_bias = tensors["o_bias"].contiguous()
         self.sink = tensors["sink"].contiguous() if self.sinks else None
         self.sink_f32 = self.sink.to(torch.float32) if self.sinks else None   # what the MFMA kernels read
         self.vmix = tensors["vmix"].reshape(1).contiguous() if self.value_mix is not None else None
@@ -164,6 +176,8 @@ class SinkAttention(Mixer):
         H, K, dk, dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
         group = ctx.groups[cache.group_id]
         proj = ops.gemm(x, self.in_proj)
+        if self.bias:
+            ops.bias_add_(proj, self.in_bias)
         inv_freq, rot_dims = self.position_encoding.frequencies() if self.position_encoding is not None else (None, 0)
         v_at = (H + K) * dk
         v_first = None
@@ -198,4 +212,6 @@ class SinkAttention(Mixer):
         if self.output_gate:
             g_at = v_at + K * dv
             ops.gated_heads(o, proj[:, g_at:g_at + H * dv], H, dv, kind=ops.GATE_SIGMOID, out=o)
+        if self.bias:
+            return ops.bias_add_(ops.gemm(o, self.o_proj), self.o_bias)
         return ops.gemm(o, self.o_proj, defer_sum=defer_sum)

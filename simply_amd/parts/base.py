@@ -109,6 +109,14 @@ class StateNeed:
         return torch.zeros((num_slots, *self.shape), dtype=self.dtype, device=device)
 
 
+@dataclasses.dataclass(frozen=True)
+class CompositeNeed:
+    """A mixer that is several mixers side by side: each keeps what its own need says.  The cache manager makes a
+    view for every part (`CacheView.parts`, in this order); needs per token join the groups of equal needs as always."""
+
+    parts: tuple
+
+
 def as_product_weight(t: torch.Tensor, shared: bool = False):
     """A matrix in the form that the matrix-product kernels read fastest: bfloat16 matrices on the GPU are
     re-laid in tiles (simply_amd/kernels/packing.py), anything else stays row-major.  `shared`: parts that are
@@ -287,13 +295,26 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class StreamPart(Part):
+    """A part at a block's end that reads and updates the residual stream itself."""
+
+    def forward(self, h: torch.Tensor, ctx: Any) -> None:
+        """h: float32 [T, D] residual stream, updated in place."""
+        raise NotImplementedError
+
+
 class Block(Part):
     """An arrangement of a mixer, a feed-forward and norms around the residual stream."""
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, norms: Mapping[str, Norm], **params):
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, norms: Mapping[str, Norm], extras=(), **params):
         self.mixer = mixer
         self.feed_forward = feed_forward
         self.norms = dict(norms)
+        #: `StreamPart`s that run on the residual stream behind the feed-forward (a block arrangement that has no
+        #: place for them refuses them)
+        self.extras = tuple(extras)
+        if self.extras and not getattr(self, "takes_extras", False):
+            raise ValueError(f"block arrangement {type(self).__name__} has no place for parts behind the feed-forward")
 
     def first_norm(self) -> Norm | None:
         """The norm that this block applies to the residual stream first, if the block before may

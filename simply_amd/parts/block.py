@@ -16,11 +16,15 @@ from .base import Block, PendingNorm
 
 @BLOCKS.register("sandwich")
 class SandwichBlock(Block):
-    NORM_NAMES = ("pre_mixer", "post_mixer", "pre_ffn", "post_ffn")
+    """A layer may have no feed-forward (its step and norms are then left out), and parts that update the residual
+    stream themselves may follow (`extras`)."""
 
-    def __init__(self, mixer, feed_forward, norms):
-        super().__init__(mixer, feed_forward, norms)
-        missing = [n for n in self.NORM_NAMES if n not in self.norms]
+    NORM_NAMES = ("pre_mixer", "post_mixer", "pre_ffn", "post_ffn")
+    takes_extras = True
+
+    def __init__(self, mixer, feed_forward, norms, extras=()):
+        super().__init__(mixer, feed_forward, norms, extras)
+        missing = [n for n in self.NORM_NAMES[:4 if feed_forward is not None else 2] if n not in self.norms]
         if missing:
             raise ValueError(f"sandwich block: norms missing: {missing}")
 
@@ -40,10 +44,19 @@ class SandwichBlock(Block):
             both = part.defers_sum and getattr(norm, "adds_partial_sums", False) and ctx.dtype == torch.bfloat16
             return {"defer_sum": True} if both else {}
 
+        # (parts behind the feed-forward change the stream once more: the next block's norm comes after them)
+        after = None if self.extras else next_norm
         y = self.mixer.forward(normed, ctx, cache, **defer(self.mixer, n["post_mixer"]))
-        normed = n["post_mixer"].add_into(h, y, n["pre_ffn"], ctx.dtype)
-        y = self.feed_forward.forward(normed, ctx, **defer(self.feed_forward, n["post_ffn"]))
-        normed_next = n["post_ffn"].add_into(h, y, next_norm, ctx.dtype)
+        if self.feed_forward is None:
+            normed_next = n["post_mixer"].add_into(h, y, after, ctx.dtype)
+        else:
+            normed = n["post_mixer"].add_into(h, y, n["pre_ffn"], ctx.dtype)
+            y = self.feed_forward.forward(normed, ctx, **defer(self.feed_forward, n["post_ffn"]))
+            normed_next = n["post_ffn"].add_into(h, y, after, ctx.dtype)
+        if self.extras:
+            for part in self.extras:
+                part.forward(h, ctx)
+            normed_next = next_norm.forward(h, ctx.dtype) if next_norm is not None else None
         return h, normed_next
 
     def _forward_few_rows(self, h, ctx, cache, normed, next_norm):
@@ -60,10 +73,19 @@ class SandwichBlock(Block):
         y = self.mixer.forward(give(self.mixer, x), ctx, cache)
         if isinstance(x, PendingNorm):
             h = x.settle()
-        x = PendingNorm(h, y, n["post_mixer"], n["pre_ffn"], ctx.dtype)
-        y = self.feed_forward.forward(give(self.feed_forward, x), ctx)
+        if self.feed_forward is None:
+            x = PendingNorm(h, y, n["post_mixer"], next_norm, ctx.dtype)
+        else:
+            x = PendingNorm(h, y, n["post_mixer"], n["pre_ffn"], ctx.dtype)
+            y = self.feed_forward.forward(give(self.feed_forward, x), ctx)
+            h = x.settle()
+            x = PendingNorm(h, y, n["post_ffn"], next_norm, ctx.dtype)
+        if not self.extras:
+            return h, x
         h = x.settle()
-        return h, PendingNorm(h, y, n["post_ffn"], next_norm, ctx.dtype)
+        for part in self.extras:
+            part.forward(h, ctx)
+        return h, PendingNorm(h, None, None, next_norm, ctx.dtype)
 
 
 @BLOCKS.register("post_norm")

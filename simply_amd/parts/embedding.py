@@ -10,7 +10,7 @@ import torch
 
 from ..kernels import ops
 from ..registry import EMBEDDINGS, HEADS
-from .base import ParamSpec, Part, as_product_weight, project
+from .base import ParamSpec, Part, StateNeed, as_product_weight, project
 
 
 @EMBEDDINGS.register("scaled_embedding")
@@ -31,6 +31,43 @@ class ScaledEmbedding(Part):
         # the factor is rounded to the table's dtype (module.py:476-480), the product is kept in float32
         scale = float(torch.tensor(self.scale, dtype=self.table.dtype))
         return ops.embed(self.table, tokens, scale)
+
+
+@EMBEDDINGS.register("summed_embedding")
+class SummedEmbedding(Part):
+    """The token's row, plus (with `pair_buckets`) a row for the pair of the token and the one before it, chosen by
+    (previous * mul_prev + token * mul_cur) mod pair_buckets, a request's first token taking the row behind the
+    buckets, plus (with `max_positions`) a learned row for the position, unscaled.  The token before a step's first
+    one is the request's state: one int32 per state slot, which this part keeps up to date."""
+
+    #: forward() takes the step's context and this part's cache view
+    needs_context = True
+
+    def __init__(self, vocab_size: int, dim: int, pair_buckets: int | None = None, mul_prev: int = 0, mul_cur: int = 0,
+                 max_positions: int | None = None):
+        self.vocab_size, self.dim = int(vocab_size), int(dim)
+        self.pair_buckets = int(pair_buckets) if pair_buckets else None
+        self.mul_prev, self.mul_cur = int(mul_prev), int(mul_cur)
+        self.max_positions = int(max_positions) if max_positions else None
+        self.table = self.pair = self.pos = None
+
+    def param_specs(self):
+        specs = {"table": ParamSpec((self.vocab_size, self.dim))}
+        if self.pair_buckets:
+            specs["pair"] = ParamSpec((self.pair_buckets + 1, self.dim))
+        if self.max_positions:
+            specs["pos"] = ParamSpec((self.max_positions, self.dim))
+        return specs
+
+    def cache_need(self):
+        return StateNeed((1,), torch.int32) if self.pair_buckets else None
+
+    def forward(self, tokens, ctx, cache):
+        if self.max_positions and ctx.max_kv_len > self.max_positions and not ctx.kv_bound:
+            raise ValueError(f"summed_embedding: a position beyond the {self.max_positions} learned ones")
+        return ops.embed_sum(tokens, ctx.positions, ctx.seq_meta, ctx.num_seqs, ctx.max_q_len, self.table,
+                             pair=self.pair, mul_prev=self.mul_prev, mul_cur=self.mul_cur,
+                             last=cache.state if cache is not None else None, pos=self.pos)
 
 
 @HEADS.register("linear_head")

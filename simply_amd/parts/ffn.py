@@ -13,6 +13,7 @@ from .base import FeedForward, ParamSpec, PendingNorm, as_product_weight, projec
 ACTIVATIONS.register("gelu_tanh", ops.ACT_GELU_TANH)
 ACTIVATIONS.register("silu", ops.ACT_SILU)
 ACTIVATIONS.register("squared_relu", ops.ACT_SQUARED_RELU)
+ACTIVATIONS.register("gelu_erf", ops.ACT_GELU_ERF)   # the exact GELU, x Phi(x)
 
 
 @FEED_FORWARDS.register("dense")
@@ -75,3 +76,55 @@ class GatedDense(FeedForward):
                 x = x.materialize()
             z = ops.gemm(x, self.gate_proj, w2=self.up_proj, activation=self.activation_code)
         return ops.gemm(z, self.down_proj, defer_sum=defer_sum)
+
+
+@FEED_FORWARDS.register("routed_experts")
+class RoutedExperts(FeedForward):
+    """A mixture of experts: `num_experts` gated feed-forwards without biases, down(act(gate x) * (up x)), of which every
+    token uses the `top` ones with the largest router scores.  Scores are the softmax of the router's logits over all
+    experts (32-bit); an expert's result is weighted by its score times `router_scale`, the weights are not renormalized.
+    With `shared_size`, one more such feed-forward runs for every token and is added, times sigmoid(w . x) (one
+    number per token) if `shared_gate`."""
+
+    def __init__(self, hidden_size: int, num_experts: int, top: int, expert_size: int, router_scale: float = 1.0,
+                 activation: str = "silu", shared_size: int | None = None, shared_gate: bool = True):
+        self.hidden_size, self.num_experts, self.top = int(hidden_size), int(num_experts), int(top)
+        self.expert_size, self.router_scale = int(expert_size), float(router_scale)
+        if not 1 <= self.top <= self.num_experts:
+            raise ValueError(f"routed_experts: top {top} of {num_experts} experts")
+        self.activation_code = int(ACTIVATIONS.get(activation))
+        self.shared = GatedDense(hidden_size, int(shared_size), activation) if shared_size else None
+        self.shared_gate = bool(shared_gate) and self.shared is not None
+        self.router = self.gate_w = self.up_w = self.down_w = None
+
+    def param_specs(self):
+        D, F, E = self.hidden_size, self.expert_size, self.num_experts
+        specs = {"router": ParamSpec((E, D))}
+        for e in range(E):
+            specs.update({f"e{e}.gate": ParamSpec((F, D)), f"e{e}.up": ParamSpec((F, D)), f"e{e}.down": ParamSpec((D, F))})
+        if self.shared is not None:
+            specs.update({"shared." + n: s for n, s in self.shared.param_specs().items()})
+            if self.shared_gate:
+                specs["shared.score"] = ParamSpec((1, D))
+        return specs
+
+    def load(self, tensors):
+        from ..kernels.packing import stack_experts
+
+        E = self.num_experts
+        rows = [tensors["router"]] + ([tensors["shared.score"]] if self.shared_gate else [])
+        # the router (and the shared expert's score) are one product, its result 32-bit
+        self.router = as_product_weight(torch.cat(rows, dim=0).contiguous())
+        self.gate_w = stack_experts(tensors[f"e{e}.gate"] for e in range(E))
+        self.up_w = stack_experts(tensors[f"e{e}.up"] for e in range(E))
+        self.down_w = stack_experts(tensors[f"e{e}.down"] for e in range(E))
+        if self.shared is not None:
+            self.shared.load({n: tensors["shared." + n] for n in self.shared.param_specs()})
+
+    def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
+        E = self.num_experts
+        logits = ops.gemm(x, self.router, out_dtype=torch.float32)
+        experts, weights = ops.route(logits[:, :E], self.top, self.router_scale)
+        shared = self.shared.forward(x, ctx) if self.shared is not None else None
+        return ops.routed_experts(x, experts, weights, self.gate_w, self.up_w, self.down_w, self.activation_code,
+                                  shared=shared, shared_gate=logits[:, E:E + 1] if self.shared_gate else None)

@@ -89,5 +89,7 @@ POSITION_ENCODINGS = Registry("position encoding")
 BLOCKS = Registry("block arrangement")
 EMBEDDINGS = Registry("embedding")
 HEADS = Registry("head")
+#: parts that read and update the residual stream themselves, behind a block's mixer and feed-forward
+STREAM_PARTS = Registry("stream part")
 #: activation name -> code of the gated product's epilogue (simply_amd/csrc/activations.h)
 ACTIVATIONS = Registry("activation")

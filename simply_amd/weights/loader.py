@@ -60,6 +60,18 @@ def weight_files(model_dir: str) -> list[str]:
     return files
 
 
+def stored_shapes(model_dir: str) -> dict[str, tuple]:
+    """Name -> shape of every tensor in the folder's files (headers only)."""
+    from safetensors import safe_open
+
+    shapes: dict[str, tuple] = {}
+    for path in weight_files(model_dir):
+        with safe_open(path, framework="pt", device="cpu") as h:
+            for name in h.keys():
+                shapes[name] = tuple(h.get_slice(name).get_shape())
+    return shapes
+
+
 def target_dtype(stored: torch.dtype, spec: ParamSpec, activation_dtype: torch.dtype) -> torch.dtype:
     if not stored.is_floating_point or spec.role == "table":
         return torch.int32
@@ -71,12 +83,12 @@ def target_dtype(stored: torch.dtype, spec: ParamSpec, activation_dtype: torch.d
 
 
 def check_names_and_shapes(where: str, expected: Mapping[str, ParamSpec], found: Mapping[str, tuple],
-                           copies: Mapping[str, str] | None = None) -> None:
+                           copies: Mapping[str, str] | None = None, ignorable=()) -> None:
     """copies: stored name -> expected tensor that it must be a copy of; such a name is not unexpected, and its
-    shape must be that tensor's."""
+    shape must be that tensor's.  ignorable: names that may be there and are left unread."""
     copies = {n: of for n, of in (copies or {}).items() if of in expected and n not in expected}
     missing = [n for n in expected if n not in found]
-    unexpected = [n for n in found if n not in expected and n not in copies]
+    unexpected = [n for n in found if n not in expected and n not in copies and n not in set(ignorable)]
     wrong = [(n, tuple(found[n]), tuple(expected[n].shape)) for n in expected
              if n in found and tuple(found[n]) != tuple(expected[n].shape)]
     wrong += [(n, tuple(found[n]), tuple(expected[of].shape)) for n, of in copies.items()
@@ -106,7 +118,7 @@ def load_weights(model, model_dir: str, activation_dtype: torch.dtype, device) -
     if duplicates:
         raise WeightsError(model_dir, [], [], [], [f"tensors stored in more than one file: {', '.join(duplicates)}"])
     copies = {n: of for n, of in getattr(model.spec, "copies", {}).items() if n in shapes and n not in expected}
-    check_names_and_shapes(model_dir, expected, shapes, copies)
+    check_names_and_shapes(model_dir, expected, shapes, copies, getattr(model.spec, "ignorable", ()))
     differing = [f"{n} is stored beside {of}, of which the model makes it a copy, but the two differ"
                  for n, of in copies.items()
                  if not torch.equal(handles[where_of[n]].get_tensor(n), handles[where_of[of]].get_tensor(of))]

@@ -115,7 +115,11 @@ def squared_relu(x):
     return torch.relu(x) ** 2
 
 
-ACTIVATIONS = (gelu_tanh, silu, squared_relu)   # by the kernels' activation codes
+def gelu_erf(x):
+    return 0.5 * x * (1.0 + torch.erf(x / math.sqrt(2.0)))
+
+
+ACTIVATIONS = (gelu_tanh, silu, squared_relu, gelu_erf)   # by the kernels' activation codes
 
 
 def gemm(a, w, *, w2=None, soft_cap=None, out_dtype=None, out=None, algo=0, shape=0, activation=0, defer_sum=False,
@@ -464,3 +468,143 @@ def score(logits, temperature, top_k, top_p, tokens, scores=None):
         scores[:R] = out
         out = scores
     return out
+
+
+# --------------------------------------------------------------------------- token tables, biases, sums of two mixers
+
+def embed_sum(tokens, positions, seq_meta, num_seqs, max_q_len, table, *, pair=None, mul_prev=0, mul_cur=0, last=None,
+              pos=None):
+    T, D = tokens.shape[0], table.shape[1]
+    out = torch.zeros((T, D), dtype=torch.float64 if PRECISE else torch.float32, device=table.device)
+    for slot, first, count, _ in seq_meta[:num_seqs].tolist():
+        for j in range(count):
+            t = first + j
+            tok, p = int(tokens[t]), int(positions[t])
+            v = _f(table[tok])
+            if pair is not None:
+                buckets = pair.shape[0] - 1
+                before = int(tokens[t - 1]) if j > 0 else int(last[slot, 0])
+                row = (before * mul_prev + tok * mul_cur) % buckets if p > 0 else buckets
+                v = v + _f(pair[row])
+            if pos is not None:
+                v = v + _f(pos[p])
+            out[t] = v
+        if pair is not None and count > 0:
+            last[slot, 0] = int(tokens[first + count - 1])
+    return out.to(torch.float32)
+
+
+def _activation(code, x):
+    return ACTIVATIONS[code](x)
+
+
+def token_gate_(z, tokens, table, col0, activation):
+    e = _f(table[tokens.long()][:, col0:col0 + z.shape[1]])
+    z.copy_((_activation(activation, _f(z)) * e).to(z.dtype))
+    return z
+
+
+def bias_add_(x, bias):
+    x.copy_((_f(x) + _f(bias)).to(x.dtype))
+    return x
+
+
+def weighted_sum(x, a, y, b, out=None):
+    r = (a * _f(x) + b * _f(y)).to(x.dtype)
+    if out is not None:
+        out.copy_(r)
+        return out
+    return r
+
+
+# --------------------------------------------------------------------------- matrix states that decay
+
+def gla_decay(u, w2, bias, tau):
+    z = _f(u) @ _f(w2).T
+    if bias is not None:
+        z = z + _f(bias)
+    return torch.exp(torch.nn.functional.logsigmoid(z) / tau).to(torch.float32)
+
+
+def exp_gates(raw, bias, cap, num_heads, m_state, seq_meta, num_seqs):
+    H = num_heads
+    x = _f(raw) + (_f(bias) if bias is not None else 0.0)
+    ig = cap * torch.tanh(x[:, :H] / cap)
+    fg = torch.nn.functional.logsigmoid(cap * torch.tanh(x[:, H:] / cap))
+    out = torch.zeros((raw.shape[0], 3 * H), dtype=x.dtype, device=raw.device)
+    for slot, first, count, _ in seq_meta[:num_seqs].tolist():
+        m = _f(m_state[slot])
+        for t in range(first, first + count):
+            new = torch.maximum(fg[t] + m, ig[t])
+            out[t, :H], out[t, H:2 * H], out[t, 2 * H:] = torch.exp(fg[t] + m - new), torch.exp(ig[t] - new), torch.exp(-new)
+            m = new
+        if count > 0:
+            m_state[slot] = m.to(torch.float32)
+    return out.to(torch.float32)
+
+
+def linear_state(proj, q_at, k_at, v_at, q_mult, gates, scalar, num_heads, key_dim, value_dim, ones, state, seq_meta,
+                 num_seqs):
+    H, dk, dv = num_heads, key_dim, value_dim
+    CT = dv + int(bool(ones))
+    T = proj.shape[0]
+    p, g = _f(proj), _f(gates)
+    out = torch.zeros((T, H * CT), dtype=p.dtype, device=proj.device)
+    for slot, first, count, _ in seq_meta[:num_seqs].tolist():
+        S = _f(state[slot, :H * dk * CT]).view(H, CT, dk).clone()   # column by column
+        for t in range(first, first + count):
+            q = p[t, q_at:q_at + H * dk].view(H, dk) * q_mult
+            k = p[t, k_at:k_at + H * dk].view(H, dk)
+            v = p[t, v_at:v_at + H * dv].view(H, dv)
+            if ones:
+                v = torch.cat([v, torch.ones((H, 1), dtype=v.dtype, device=v.device)], dim=1)
+            if scalar:
+                a, c = g[t, :H].view(H, 1, 1), g[t, H:2 * H].view(H, 1)
+            else:
+                a, c = g[t, :H * dk].view(H, 1, dk), 1.0
+            S = a * S + (c * v)[:, :, None] * k[:, None, :]
+            out[t] = torch.einsum("hcd,hd->hc", S, q).reshape(-1)
+        if count > 0:
+            state[slot, :H * dk * CT] = S.reshape(-1).to(torch.float32)
+    return out.to(torch.float32)
+
+
+def normalized_readout(x, floor, gate, weight, eps, num_heads, size, out_dtype):
+    T, H = x.shape[0], num_heads
+    xs = _f(x).view(T, H, size + 1)
+    o = xs[:, :, :size] / (torch.maximum(xs[:, :, size:].abs(), _f(floor)[:, :, None]) + 1e-6)
+    o = o * torch.rsqrt((o * o).mean(-1, keepdim=True) + eps)
+    o = o.reshape(T, H * size) * _f(weight) * torch.sigmoid(_f(gate))
+    return o.to(out_dtype)
+
+
+# --------------------------------------------------------------------------- routed experts
+
+def route(logits, top, scale):
+    s = torch.softmax(_f(logits), -1)
+    best = torch.topk(s, top, dim=-1)
+    return best.indices.to(torch.int32).contiguous(), (best.values * scale).to(torch.float32).contiguous()
+
+
+def routed_experts(x, experts, weights, gate_w, up_w, down_w, activation, *, shared=None, shared_gate=None,
+                   out_dtype=None):
+    from simply_amd.kernels.packing import TiledWeight, unpack_tiles
+
+    def matrix(stack, e):
+        if stack.tiled:
+            return _f(unpack_tiles(TiledWeight(stack.data[e], stack.rows, stack.cols)))
+        return _f(stack.data[e])
+
+    T, D = x.shape
+    xf = _f(x)
+    out = torch.zeros((T, D), dtype=xf.dtype, device=x.device)
+    for t in range(T):
+        for k in range(experts.shape[1]):
+            e = int(experts[t, k])
+            h = _activation(activation, (xf[t] @ matrix(gate_w, e).T).to(x.dtype).to(xf.dtype)) \
+                * (xf[t] @ matrix(up_w, e).T).to(x.dtype).to(xf.dtype)
+            out[t] += _f(weights[t, k]) * (h.to(x.dtype).to(xf.dtype) @ matrix(down_w, e).T)
+    if shared is not None:
+        s = _f(shared)
+        out = out + (s * torch.sigmoid(_f(shared_gate)[:, :1]) if shared_gate is not None else s)
+    return out.to(out_dtype or x.dtype)
