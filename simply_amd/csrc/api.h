@@ -392,15 +392,16 @@ int sa_normalized_readout(const float* x, const float* floor, int64_t floor_stri
 // softmax over E logits, the top largest: experts [T, top], weights [T, top] = score * scale.
 int sa_route(const float* logits, int64_t stride, int T, int E, int top, float scale, int* experts, float* weights,
              hipStream_t stream);
-// The most tiles of 16 rows of one expert that P pairs over E experts make.
-int sa_expert_tiles_max(int P, int E);
-// sorted [P]: the pairs by expert; plan [1 + 2 * sa_expert_tiles_max(P, E)]: the tiles.
-int sa_expert_sort(const int* experts, int P, int E, int* sorted, int* plan, int plan_words, hipStream_t stream);
+// The most tiles of tile_rows (16 or 64) rows of one expert that P pairs over E experts make.
+int sa_expert_tiles_max(int P, int E, int tile_rows);
+// sorted [P]: the pairs by expert; plan [1 + 2 * sa_expert_tiles_max(P, E, tile_rows)]: the tiles.
+int sa_expert_sort(const int* experts, int P, int E, int tile_rows, int* sorted, int* plan, int plan_words,
+                   hipStream_t stream);
 // w2 given: out[row] = act(a . w1[e]^T) * (a . w2[e]^T) in a's type; else out[row] = a . w1[e]^T in 32-bit.  a's row is
 // the pair's token (a_by_token) or its place in the sorted order; out's row the pair (out_by_pair) or that place.
 // bfloat16 weights are tiled [E][ceil(N / 16)][ceil(K / 32)][64][8], 32-bit ones row-major [E][N][K].
 int sa_expert_product(const void* a, int dtype, int64_t a_stride, int a_by_token, int top, const void* w1, const void* w2,
-                      int N, int K, const int* sorted, const int* plan, int P, int E, int act, void* out,
+                      int N, int K, const int* sorted, const int* plan, int P, int E, int tile_rows, int act, void* out,
                       int64_t out_stride, int out_by_pair, hipStream_t stream);
 // out[t] = sum_k weights[t, k] y[t * top + k] + sigmoid(gate[t]) * shared[t]  (shared null: none; gate null: 1).
 int sa_expert_combine(const float* y, const float* weights, int top, const void* shared, int shared_dtype,

@@ -2,8 +2,8 @@
 //
 //   route_kernel          softmax of the router's logits, the `top` largest scores and their experts
 //   sort_kernel           the (token, choice) pairs in the order of their experts, cut into tiles of rows of one expert
-//   expert_gate_up_kernel h = act(Wg[e] x) * (Wu[e] x) for every pair, rows in the sorted order
-//   expert_down_kernel    y = Wd[e] h, one row per pair (in the pairs' own order)
+//   expert_product_kernel h = act(Wg[e] x) * (Wu[e] x) for every pair, rows in the sorted order; then
+//                         y = Wd[e] h, one row per pair (in the pairs' own order)
 //   combine_kernel        out[t] = sum_k weight[t, k] y[t, k] + sigmoid(s[t]) * shared[t]
 //
 // Nothing comes back to the host between them: the tiles are found on the device, and the grid of the expert
@@ -16,7 +16,7 @@
 namespace sa {
 
 constexpr int kRouteSlots = 8;    // experts per lane: up to 512 experts
-constexpr int kTileRows = 16;     // rows of a tile: one MFMA operand
+constexpr int kTileRowsMax = 64;  // rows of a tile: 16 (one MFMA operand) or 64 (four, which share the weights' operands)
 
 // A wave per token.  scores = softmax(logits); `top` times the largest score that is left (of equal ones the lowest
 // index); weight = score * scale.
@@ -62,9 +62,10 @@ __global__ __launch_bounds__(kWave) void route_kernel(const float* __restrict__ 
 }
 
 // One workgroup.  plan: [0] number of tiles; [1 .. 1 + 2 * max_tiles): per tile its expert and its first row in the
-// sorted order with the number of its rows packed as first * 32 + rows.  sorted [P]: pair indices by expert.
+// sorted order with the number of its rows packed as first * 128 + rows.  sorted [P]: pair indices by expert.
 __global__ __launch_bounds__(1024) void sort_kernel(const int* __restrict__ experts, int P, int E,
-                                                    int* __restrict__ sorted, int* __restrict__ plan, int max_tiles) {
+                                                    int* __restrict__ sorted, int* __restrict__ plan, int max_tiles,
+                                                    int kTileRows) {
   extern __shared__ int lds[];   // counts [E], offsets [E + 1], tile offsets [E + 1], cursors [E]
   int* counts = lds;
   int* offsets = lds + E;
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(1024) void sort_kernel(const int* __restrict__ expe
       if (n >= max_tiles) break;
       const int rows = counts[e] - i * kTileRows < kTileRows ? counts[e] - i * kTileRows : kTileRows;
       plan[1 + 2 * n] = e;
-      plan[2 + 2 * n] = (offsets[e] + i * kTileRows) * 32 + rows;
+      plan[2 + 2 * n] = (offsets[e] + i * kTileRows) * 128 + rows;
     }
   }
   __syncthreads();
@@ -111,10 +112,11 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 __device__ __forceinline__ bf16x8 load8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
 // h[row, f] = act(x[token] . Wg[e, f]) * (x[token] . Wu[e, f]); GATED false: y[pair, n] = h[row] . Wd[e, n].
-// A workgroup of four waves takes one tile of rows and 64 columns (a wave 16 of them).
+// A workgroup of four waves takes one tile of rows and 64 columns (a wave 16 of them, for all RT sub-tiles of 16 rows).
 // bfloat16: the weights are tiled ([E][N / 16][K / 32][64][8], see the product kernels), a wave's operands are one
-// 16-byte load a lane; 32-bit: row-major weights [E][N][K], a lane per (row, column) of the tile in turn.
-template <typename T, bool GATED>
+// 16-byte load a lane (rows that are not 16-byte aligned are read element by element); 32-bit: row-major weights
+// [E][N][K], a lane per (row, column) of the tile in turn.
+template <typename T, bool GATED, int RT>
 __global__ __launch_bounds__(256) void expert_product_kernel(
     const T* __restrict__ a, int64_t a_stride, int a_by_token, int top, const T* __restrict__ w1, const T* __restrict__ w2,
     int N, int K, const int* __restrict__ sorted, const int* __restrict__ plan, int act, void* __restrict__ out,
@@ -122,52 +124,70 @@ __global__ __launch_bounds__(256) void expert_product_kernel(
   const int tile = blockIdx.x;
   if (tile >= plan[0]) return;
   const int e = plan[1 + 2 * tile], packed = plan[2 + 2 * tile];
-  const int row0 = packed / 32, rows = packed % 32;
+  const int row0 = packed / 128, rows = packed % 128;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int n0 = (blockIdx.y * 4 + wave) * 16;
   if (n0 >= N) return;
   if constexpr (sizeof(T) == 2) {
     const int Nt = (N + 15) / 16, Kt = (K + 31) / 32;
     const int r = lane % 16, kq = lane / 16;
-    const int rr = r < rows ? r : rows - 1;
-    const int pair = sorted[row0 + rr];
-    const T* arow = a + static_cast<size_t>(a_by_token ? pair / top : row0 + rr) * a_stride;
+    const bool aligned = a_stride % 8 == 0;
+    const T* arow[RT];
+    int pairs[RT];
+#pragma unroll
+    for (int s = 0; s < RT; ++s) {
+      const int rr = s * 16 + r < rows ? s * 16 + r : rows - 1;
+      pairs[s] = sorted[row0 + rr];
+      arow[s] = a + static_cast<size_t>(a_by_token ? pairs[s] / top : row0 + rr) * a_stride;
+    }
     const size_t wbase = (static_cast<size_t>(e) * Nt + n0 / 16) * Kt;
     const bf16* g = reinterpret_cast<const bf16*>(w1) + wbase * 512 + lane * 8;
     const bf16* u = GATED ? reinterpret_cast<const bf16*>(w2) + wbase * 512 + lane * 8 : nullptr;
-    floatx4 accg = {0.f, 0.f, 0.f, 0.f}, accu = {0.f, 0.f, 0.f, 0.f};
+    floatx4 accg[RT], accu[RT];
+#pragma unroll
+    for (int s = 0; s < RT; ++s) accg[s] = accu[s] = floatx4{0.f, 0.f, 0.f, 0.f};
     for (int kt = 0; kt < Kt; ++kt) {
       const int k = kt * 32 + kq * 8;
-      bf16x8 av;
-      if (k + 8 <= K) {
-        av = load8(reinterpret_cast<const bf16*>(arow) + k);
-      } else {
+      const bf16x8 gv = load8(g + static_cast<size_t>(kt) * 512);
+      bf16x8 uv = gv;
+      if constexpr (GATED) uv = load8(u + static_cast<size_t>(kt) * 512);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) av[i] = k + i < K ? __builtin_bit_cast(__bf16, reinterpret_cast<const bf16*>(arow)[k + i]) : static_cast<__bf16>(0.f);
+      for (int s = 0; s < RT; ++s) {
+        if (s * 16 >= rows) break;   // (uniform: the tile's rows are)
+        const bf16* src = reinterpret_cast<const bf16*>(arow[s]);
+        bf16x8 av;
+        if (aligned && k + 8 <= K) {
+          av = load8(src + k);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i)
+            av[i] = k + i < K ? __builtin_bit_cast(__bf16, src[k + i]) : static_cast<__bf16>(0.f);
+        }
+        // the weights' rows are the product's columns: C^T = W . A^T, a lane holds four columns of the output of
+        // one token
+        accg[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gv, av, accg[s], 0, 0, 0);
+        if constexpr (GATED) accu[s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uv, av, accu[s], 0, 0, 0);
       }
-      // the weights' rows are the product's columns: C^T = W . A^T, a lane holds four rows (columns of the
-      // output) of one token
-      accg = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load8(g + static_cast<size_t>(kt) * 512), av, accg, 0, 0, 0);
-      if constexpr (GATED)
-        accu = __builtin_amdgcn_mfma_f32_16x16x32_bf16(load8(u + static_cast<size_t>(kt) * 512), av, accu, 0, 0, 0);
     }
-    // lane: token r = lane % 16, output columns n0 + kq * 4 + i
-    if (r < rows) {
-      const size_t orow = static_cast<size_t>(out_by_pair ? pair : row0 + r) * out_stride;
+    // lane: token s * 16 + lane % 16, output columns n0 + kq * 4 + i
+#pragma unroll
+    for (int s = 0; s < RT; ++s) {
+      if (s * 16 + r >= rows) continue;
+      const size_t orow = static_cast<size_t>(out_by_pair ? pairs[s] : row0 + s * 16 + r) * out_stride;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int n = n0 + kq * 4 + i;
         if (n >= N) continue;
         if constexpr (GATED) {
-          const float v = gated_activation(act, to_float(float_to_bf16(accg[i]))) * to_float(float_to_bf16(accu[i]));
+          const float v = gated_activation(act, to_float(float_to_bf16(accg[s][i]))) * to_float(float_to_bf16(accu[s][i]));
           static_cast<bf16*>(out)[orow + n] = float_to_bf16(v);
         } else {
-          static_cast<float*>(out)[orow + n] = accg[i];
+          static_cast<float*>(out)[orow + n] = accg[s][i];
         }
       }
     }
   } else {
-    // 32-bit: 16 columns x up to 16 rows of the tile over the wave's 64 lanes, four rows a lane
+    // 32-bit: 16 columns x the rows of the tile over the wave's 64 lanes, four rows at a time
     const int c = lane % 16, n = n0 + c;
     for (int r = lane / 16; r < rows; r += 4) {
       const int pair = sorted[row0 + r];
@@ -219,23 +239,27 @@ extern "C" int sa_route(const float* logits, int64_t stride, int T, int E, int t
   return check_launch("route");
 }
 
-extern "C" int sa_expert_tiles_max(int P, int E) { return (P + kTileRows - 1) / kTileRows + (E < P ? E : P); }
+extern "C" int sa_expert_tiles_max(int P, int E, int tile_rows) {
+  return (P + tile_rows - 1) / tile_rows + (E < P ? E : P);
+}
 
-extern "C" int sa_expert_sort(const int* experts, int P, int E, int* sorted, int* plan, int plan_words,
+extern "C" int sa_expert_sort(const int* experts, int P, int E, int tile_rows, int* sorted, int* plan, int plan_words,
                               hipStream_t stream) {
   if (P == 0) return 0;
-  const int max_tiles = sa_expert_tiles_max(P, E);
+  SA_REQUIRE(tile_rows == 16 || tile_rows == kTileRowsMax, "expert_sort: tiles of 16 or %d rows", kTileRowsMax);
+  const int max_tiles = sa_expert_tiles_max(P, E, tile_rows);
   SA_REQUIRE(P > 0 && E > 0 && E <= 4096 && P < (1 << 26), "expert_sort: bad sizes P=%d E=%d", P, E);
   SA_REQUIRE(plan_words >= 1 + 2 * max_tiles, "expert_sort: the plan needs %d words", 1 + 2 * max_tiles);
   SA_REQUIRE(experts != nullptr && sorted != nullptr && plan != nullptr, "expert_sort: a null pointer");
   const int threads = P >= 1024 ? 1024 : ((P + kWave - 1) / kWave) * kWave;
-  sort_kernel<<<1, threads, (4 * E + 2) * sizeof(int), stream>>>(experts, P, E, sorted, plan, max_tiles);
+  sort_kernel<<<1, threads, (4 * E + 2) * sizeof(int), stream>>>(experts, P, E, sorted, plan, max_tiles, tile_rows);
   return check_launch("expert_sort");
 }
 
 extern "C" int sa_expert_product(const void* a, int dtype, int64_t a_stride, int a_by_token, int top, const void* w1,
-                                 const void* w2, int N, int K, const int* sorted, const int* plan, int P, int E, int act,
-                                 void* out, int64_t out_stride, int out_by_pair, hipStream_t stream) {
+                                 const void* w2, int N, int K, const int* sorted, const int* plan, int P, int E,
+                                 int tile_rows, int act, void* out, int64_t out_stride, int out_by_pair,
+                                 hipStream_t stream) {
   if (P == 0) return 0;
   SA_REQUIRE(P > 0 && E > 0 && N > 0 && K > 0 && top > 0 && a_stride >= K && out_stride >= N,
              "expert_product: bad sizes P=%d E=%d N=%d K=%d", P, E, N, K);
@@ -243,20 +267,25 @@ extern "C" int sa_expert_product(const void* a, int dtype, int64_t a_stride, int
              "expert_product: a null pointer");
   SA_REQUIRE(act >= 0 && act < kNumActivations, "expert_product: unknown activation %d", act);
   SA_REQUIRE(dtype == kF32 || dtype == kBF16, "expert_product: unknown dtype %d", dtype);
-  SA_REQUIRE(dtype == kF32 || (a_stride % 8 == 0), "expert_product: bfloat16 rows must be 16-byte aligned");
-  const dim3 grid(sa_expert_tiles_max(P, E), (N + 63) / 64);
+  SA_REQUIRE(tile_rows == 16 || tile_rows == kTileRowsMax, "expert_product: tiles of 16 or %d rows", kTileRowsMax);
+  const dim3 grid(sa_expert_tiles_max(P, E, tile_rows), (N + 63) / 64);
   SA_REQUIRE(grid.y <= 65535, "expert_product: too many columns");
   const bool gated = w2 != nullptr;
-#define SA_EXPERT(T, G)                                                                                                \
-  expert_product_kernel<T, G><<<grid, 256, 0, stream>>>(static_cast<const T*>(a), a_stride, a_by_token, top,            \
-                                                         static_cast<const T*>(w1), static_cast<const T*>(w2), N, K,   \
-                                                         sorted, plan, act, out, out_stride, out_by_pair)
+#define SA_EXPERT(T, G, RT)                                                                                            \
+  expert_product_kernel<T, G, RT><<<grid, 256, 0, stream>>>(static_cast<const T*>(a), a_stride, a_by_token, top,        \
+                                                             static_cast<const T*>(w1), static_cast<const T*>(w2), N,  \
+                                                             K, sorted, plan, act, out, out_stride, out_by_pair)
   if (dtype == kBF16) {
-    if (gated) SA_EXPERT(bf16, true);
-    else SA_EXPERT(bf16, false);
+    if (tile_rows == 16) {
+      if (gated) SA_EXPERT(bf16, true, 1);
+      else SA_EXPERT(bf16, false, 1);
+    } else {
+      if (gated) SA_EXPERT(bf16, true, 4);
+      else SA_EXPERT(bf16, false, 4);
+    }
   } else {
-    if (gated) SA_EXPERT(float, true);
-    else SA_EXPERT(float, false);
+    if (gated) SA_EXPERT(float, true, 1);
+    else SA_EXPERT(float, false, 1);
   }
 #undef SA_EXPERT
   return check_launch("expert_product");

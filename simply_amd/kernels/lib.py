@@ -78,8 +78,8 @@ _SIGNATURES = {
     "sa_linear_state": [_P, _I, _L, _I, _I, _I, _F, _P, _L, _I, _I, _I, _I, _I, _P, _L, _P, _I, _P, _P],
     "sa_normalized_readout": [_P, _P, _L, _P, _I, _L, _P, _I, _F, _P, _I, _L, _I, _I, _I, _P],
     "sa_route": [_P, _L, _I, _I, _I, _F, _P, _P, _P],
-    "sa_expert_sort": [_P, _I, _I, _P, _P, _I, _P],
-    "sa_expert_product": [_P, _I, _L, _I, _I, _P, _P, _I, _I, _P, _P, _I, _I, _I, _P, _L, _I, _P],
+    "sa_expert_sort": [_P, _I, _I, _I, _P, _P, _I, _P],
+    "sa_expert_product": [_P, _I, _L, _I, _I, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _P, _L, _I, _P],
     "sa_expert_combine": [_P, _P, _I, _P, _I, _L, _P, _L, _P, _I, _L, _I, _I, _P],
     "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _L, _P],
 }
@@ -120,7 +120,7 @@ def load() -> ctypes.CDLL:
             fn.restype = c_int
         lib.sa_gemm_plan.argtypes = [_I, _I, _I, _I, _I, _L, _P]
         lib.sa_gemm_plan.restype = c_int
-        lib.sa_expert_tiles_max.argtypes = [_I, _I]
+        lib.sa_expert_tiles_max.argtypes = [_I, _I, _I]
         lib.sa_expert_tiles_max.restype = c_int
         lib.sa_philox4x32_10.argtypes = [_P, _P, _P]
         lib.sa_philox4x32_10.restype = None

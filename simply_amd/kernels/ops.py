@@ -1234,16 +1234,18 @@ def routed_experts(x: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor
         raise KernelError("routed_experts: experts int32 [T, top] and weights float32 [T, top] expected")
     P = T * top
     dev = x.device
-    max_tiles = _lib.load().sa_expert_tiles_max(P, E)
+    # tiles of 64 rows share the weights' operands between four sub-tiles: for steps that bring an expert many rows
+    tile_rows = 64 if P >= 32 * E else 16
+    max_tiles = _lib.load().sa_expert_tiles_max(P, E, tile_rows)
     sorted_ = torch.empty(P, dtype=torch.int32, device=dev)
     plan = torch.empty(1 + 2 * max_tiles, dtype=torch.int32, device=dev)
-    _lib.call("sa_expert_sort", _ptr(experts), P, E, _ptr(sorted_), _ptr(plan), plan.numel(), _stream())
+    _lib.call("sa_expert_sort", _ptr(experts), P, E, tile_rows, _ptr(sorted_), _ptr(plan), plan.numel(), _stream())
     h = torch.empty((P, F), dtype=x.dtype, device=dev)
     _lib.call("sa_expert_product", _ptr(x), _code(x), _rows(x, "routed_experts: x"), 1, top, _ptr(gate_w.data),
-              _ptr(up_w.data), F, D, _ptr(sorted_), _ptr(plan), P, E, int(activation), _ptr(h), F, 0, _stream())
+              _ptr(up_w.data), F, D, _ptr(sorted_), _ptr(plan), P, E, tile_rows, int(activation), _ptr(h), F, 0, _stream())
     y = torch.empty((P, D), dtype=torch.float32, device=dev)
     _lib.call("sa_expert_product", _ptr(h), _code(h), F, 0, top, _ptr(down_w.data), None, D, F, _ptr(sorted_), _ptr(plan), P,
-              E, 0, _ptr(y), D, 1, _stream())
+              E, tile_rows, 0, _ptr(y), D, 1, _stream())
     out = torch.empty((T, D), dtype=out_dtype or x.dtype, device=dev)
     if shared is not None and tuple(shared.shape) != (T, D):
         raise KernelError("routed_experts: the shared expert's rows do not match")

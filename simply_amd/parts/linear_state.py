@@ -22,11 +22,14 @@ import torch
 
 from ..kernels import ops
 from ..registry import MIXERS
-from .base import Mixer, ParamSpec, StateNeed, as_product_weight
+from .base import Mixer, ParamSpec, StateNeed, as_product_weight, project
 
 
 @MIXERS.register("gated_linear_attention")
 class GatedLinearAttention(Mixer):
+    #: the mixer's input enters one product only: for a few rows the norm in front of it runs in that product's kernel
+    accepts_pending = True
+
     def __init__(self, hidden_size: int, num_heads: int, key_dim: int, value_dim: int, decay_rank: int, tau: float,
                  norm_eps: float):
         self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
@@ -64,7 +67,7 @@ class GatedLinearAttention(Mixer):
         C = H * dk
         g_at = 2 * C + H * dv
         u_at = g_at + H * dv
-        proj = ops.gemm(x, self.in_proj)
+        proj = project(x, self.in_proj)
         decay = ops.gla_decay(proj[:, u_at:u_at + R], self.decay_out, self.decay_bias, self.tau)
         o = ops.linear_state(proj, 0, C, 2 * C, dk ** -0.5, decay, False, H, dk, dv, False, cache.state, ctx.seq_meta,
                              ctx.num_seqs)

@@ -213,3 +213,19 @@ def greedy(w, cfg, prompt, steps, dtype=torch.float64):
     for _ in range(steps):
         tokens.append(int(forward(w, cfg, tokens, dtype)[-1].argmax()))
     return tokens[len(prompt):]
+
+
+def load(model_dir: str):
+    """(weights by tensor name as stored, config.json as a dict)."""
+    import json
+    import os
+
+    from safetensors import safe_open
+
+    with open(os.path.join(model_dir, "config.json")) as f:
+        cfg = json.load(f)
+    w = {}
+    with safe_open(os.path.join(model_dir, "model.safetensors"), framework="pt", device="cpu") as h:
+        for name in h.keys():
+            w[name] = h.get_tensor(name)
+    return w, cfg

@@ -1,0 +1,139 @@
+"""Nemidra without a GPU: configuration and weights, the plain implementation's own invariants, and the engine's host
+logic (cache needs of several parts, the loop over layers, the embedding's state) with the kernels replaced by their
+plain torch references."""
+import copy
+
+import pytest
+import torch
+
+import nemidra_cases as cases
+import nemidra_mechanisms as mech
+import plain_nemidra as plain
+from simply_amd.config import ConfigError, NemidraConfig, config_from_dict, load_config
+from simply_amd.models import DecoderModel
+from simply_amd.weights import WeightsError, load_weights
+
+CPU = "cpu"
+
+
+def test_config_and_schedule():
+    cfg = config_from_dict(cases.MIXED)
+    assert isinstance(cfg, NemidraConfig) and cfg.to_dict() == cases.MIXED
+    spec = cfg.model_spec()
+    assert [(e.layer, e.add_embedding) for e in spec.schedule] == \
+        [(0, False), (1, False), (2, False), (1, True), (2, False), (1, True), (2, False), (3, False)]
+    assert [(e.layer, e.add_embedding) for e in config_from_dict(cases.LOOP_FROM_START).model_spec().schedule] == \
+        [(0, False), (1, False), (0, True), (1, False)]
+    assert [e.layer for e in config_from_dict(cases.UNITS).model_spec().schedule] == [0, 1, 2]
+    model = DecoderModel(spec)
+    names = set(model.expected_tensors())
+    assert {"embed", "bigram", "pos", "side.embed", "l0.mix.a2.b", "l1.mix.left.q.b", "l1.mix.right.f.b", "l1.mlp.e4.down",
+            "l1.mlp.shared.sg", "l2.mlp.router", "l3.side.norm", "final.norm", "head"} <= names
+    assert "l3.norm2" not in names and "l2.mlp.shared.gate" not in names
+    # every pass of the loop has a cache or a state of its own; the embedding's state comes last
+    needs = model.cache_needs()
+    assert len(needs) == len(spec.schedule) + 1 and all(c is None for _, c in needs)
+
+
+@pytest.mark.parametrize("change, message", [
+    (lambda d: d["layers"][0].update(type="conv"), "unknown layer type"),
+    (lambda d: d["layers"][0]["mixer"].pop("rank"), "rank"),
+    (lambda d: d["layers"][1]["mixer"]["left"].pop("scale"), "scale"),
+    (lambda d: d["layers"][1]["mlp"].update(kind="sparse"), "unknown kind"),
+    (lambda d: d["loop"].update(stop=9), "loop"),
+    (lambda d: d["loop"].update(times=0), "loop"),
+    (lambda d: d.pop("vocab"), "vocab"),
+])
+def test_config_errors(change, message):
+    d = copy.deepcopy(cases.MIXED)
+    change(d)
+    with pytest.raises((ConfigError, ValueError), match=message):
+        config_from_dict(d)
+
+
+def test_folder_round_trip_rank_from_the_tensor_and_tolerated_norms(tmp_path):
+    """A folder whose config.json does not say the decay's rank: the tensor's shape does.  Norms of a feed-forward that a
+    layer does not have may be stored and are left unread; anything else that is unexpected is an error."""
+    import json
+    import os
+
+    from safetensors.torch import load_file, save_file
+
+    d = cases.write_model("mixed", str(tmp_path / "m"))
+    path = os.path.join(d, "config.json")
+    raw = json.load(open(path))
+    for l in raw["layers"]:
+        l["mixer"].pop("rank", None)
+    json.dump(raw, open(path, "w"))
+    cfg = load_config(d)
+    assert cfg.model_spec().layers[0].mixer.params["decay_rank"] == 5
+    tensors = load_file(os.path.join(d, "model.safetensors"))
+    tensors["l3.norm2"] = torch.zeros(40)
+    save_file(tensors, os.path.join(d, "model.safetensors"))
+    model = DecoderModel(cfg.model_spec())
+    load_weights(model, d, torch.float32, torch.device("cpu"))
+    tensors["l3.norm3"] = torch.zeros(40)
+    del tensors["l0.mix.a2.b"]
+    save_file(tensors, os.path.join(d, "model.safetensors"))
+    with pytest.raises(WeightsError) as e:
+        load_weights(DecoderModel(cfg.model_spec()), d, torch.float32, torch.device("cpu"))
+    assert e.value.missing == ["l0.mix.a2.b"] and e.value.unexpected == ["l3.norm3"]
+
+
+def test_plain_recurrences_in_portions():
+    """The plain recurrences are their own check: the matrix memory computed with the running maximum equals the one
+    computed without it (in float64, where nothing overflows at these sizes)."""
+    g = torch.Generator().manual_seed(0)
+    T, D, H, dk, dv = 30, 16, 2, 4, 6
+    w = {"p." + n: torch.randn(*s, generator=g, dtype=torch.float64) * 0.4 for n, s in
+         dict(q=(H * dk, D), k=(H * dk, D), v=(H * dv, D), g=(H * dv, D), o=(D, H * dv), i=(H, D), f=(H, D)).items()}
+    w |= {"p.i.b": torch.zeros(H, dtype=torch.float64), "p.f.b": torch.ones(H, dtype=torch.float64),
+          "p.norm": torch.ones(H * dv, dtype=torch.float64)}
+    h = torch.randn(T, D, generator=g, dtype=torch.float64)
+    m = {"heads": H, "dim": dk, "vdim": dv, "gate_cap": 15.0}
+    got = plain.mlstm(w, "p.", m, h, 1e-6)
+    q = (h @ w["p.q"].T).view(T, H, dk) * dk ** -0.5
+    k, v = (h @ w["p.k"].T).view(T, H, dk), (h @ w["p.v"].T).view(T, H, dv)
+    ig = 15.0 * torch.tanh((h @ w["p.i"].T) / 15.0)
+    fg = torch.nn.functional.logsigmoid(15.0 * torch.tanh((h @ w["p.f"].T + 1.0) / 15.0))
+    out = torch.zeros(T, H, dv, dtype=torch.float64)
+    for a in range(H):
+        S, n, logm = torch.zeros(dk, dv, dtype=torch.float64), torch.zeros(dk, dtype=torch.float64), 0.0
+        for t in range(T):   # unscaled: S holds the true sums, the floor is exp(-m) * exp(m) = 1 in these units
+            S = torch.exp(fg[t, a]) * S + torch.exp(ig[t, a]) * torch.outer(k[t, a], v[t, a])
+            n = torch.exp(fg[t, a]) * n + torch.exp(ig[t, a]) * k[t, a]
+            logm = max(float(fg[t, a]) + logm, float(ig[t, a]))
+            scale = torch.exp(torch.tensor(-logm, dtype=torch.float64))
+            out[t, a] = (S.T @ q[t, a]) * scale / (torch.maximum((n @ q[t, a]).abs() * scale, scale) + 1e-6)
+    want = (plain.rms_unit(out, 1e-6).reshape(T, H * dv) * torch.sigmoid(h @ w["p.g"].T)) @ w["p.o"].T
+    assert float((got - want).abs().max()) < 1e-9
+
+
+@pytest.mark.parametrize("body", [mech.gla_part, mech.memory_part, mech.window_edges, mech.far_key_without_window,
+                                  mech.parallel_part, mech.routed_experts_part, mech.dense_part, mech.embedding_part,
+                                  mech.token_side_part])
+def test_part(cpu_ops, body):
+    body(CPU, torch.float32)
+
+
+@pytest.mark.parametrize("name", ["mixed", "units", "loop_from_start"])
+def test_cuts_match_plain(tmp_path, cpu_ops, name):
+    cases.cuts_match_plain(tmp_path, CPU, name)
+
+
+@pytest.mark.parametrize("name", ["mixed", "units"])
+def test_batches_match_alone(tmp_path, cpu_ops, name):
+    cases.batches_match_alone(tmp_path, CPU, name)
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+def test_drawn_configurations(tmp_path, cpu_ops, seed):
+    cases.drawn_configuration_runs(tmp_path, CPU, seed)
+
+
+def test_layers_match_plain(tmp_path, cpu_ops):
+    cases.layers_match_plain(tmp_path, CPU)
+
+
+def test_greedy_generation(tmp_path, cpu_ops):
+    cases.greedy_generation(tmp_path, CPU)
