@@ -448,6 +448,55 @@ def run_zenuzen(args):
             torch.cuda.empty_cache()
 
 
+# --only nemidra: layer sizes that resemble a real model's, for the Nemidra design (three layers of gated linear
+# attention to one with windowed attention beside a matrix memory; dense feed-forwards and routed experts in turn, the
+# routed ones with about as many active parameters as the dense ones; pair and position tables, the per-layer token
+# input) and, beside it, the closest model that the engine has, Zenuzen, at equal width, depth, heads and head size
+def nemidra_config(size: dict, layers: int, positions: int) -> dict:
+    W, H, K, d, ff = size["width"], size["heads"], size["kv_heads"], size["dim"], size["ff"]
+    out = []
+    for i in range(layers):
+        if i % 2 == 0:
+            mlp = {"kind": "dense", "ff": ff}
+        else:
+            mlp = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 16, "top": 2, "scale": 1.0},
+                   "shared": {"ff": ff // 4}}
+        if i % 4 == 3:
+            mixer = {"left": {"heads": H, "kv_heads": K, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024}},
+                     "right": {"heads": H // 2, "dim": d, "vdim": d, "gate_cap": 15.0}, "left_scale": 1.0, "right_scale": 1.0}
+            out.append({"type": "parallel", "mixer": mixer, "mlp": mlp})
+        else:
+            out.append({"type": "gla", "mixer": {"heads": H, "dim": d, "vdim": d, "tau": 16.0, "rank": 64}, "mlp": mlp})
+    return {"architecture": "Nemidra", "vocab": size["vocab"], "width": W, "norm": {"eps": 1e-5}, "layers": out,
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}, "max_positions": positions,
+            "token_side": {"dim": 64}, "logit_softcap": 30.0}
+
+
+def run_nemidra(args):
+    import torch
+    from simply_amd.config import config_from_dict
+    from simply_amd.engine.loading import random_model
+
+    tdtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    layers = args.layers or 8
+    positions = max(args.prefill_tokens, args.context + args.steps + args.warmup) + 16
+    for name in args.sizes.split(","):
+        size = ZENUZEN_SIZES[name]
+        for label, d in (("nemidra", nemidra_config(size, layers, positions)), ("zenuzen-equal-size", zenuzen_config(size, layers))):
+            cfg = config_from_dict(d)
+            model = random_model(cfg, 0, tdtype, torch.device("cuda:0"), std=0.02)
+            pt, dt = run_executor_bench(model, size["vocab"], args.prefill_tokens, args.batch, args.context, args.steps,
+                                        args.warmup, args.page_size, args.dtype)
+            print(json.dumps({"metric": "prefill and decode tokens/s through the step function", "model": label,
+                              "size": name, "width": size["width"], "layers": layers,
+                              "prefill_tokens": args.prefill_tokens, "prefill_tokens_per_s": round(args.prefill_tokens / pt, 1),
+                              "prefill_ms": round(pt * 1e3, 3), "batch": args.batch, "context": args.context,
+                              "decode_tokens_per_s": round(args.batch / dt, 1), "decode_ms_per_step": round(dt * 1e3, 3),
+                              "dtype": args.dtype, "data": "synthetic"}), flush=True)
+            del model
+            torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -463,7 +512,7 @@ def main():
     ap.add_argument("--batches", default="1,8,32,64", help="--only decode-grid: the batch sizes")
     ap.add_argument("--contexts", default="1024,4096,8192", help="--only decode-grid: the context lengths")
     ap.add_argument("--only", default="all", choices=["all", "decode", "decode-grid", "prefill", "prefill-chunked", "products",
-                                                      "gated-products", "ceilings", "zenuzen"],
+                                                      "gated-products", "ceilings", "zenuzen", "nemidra"],
                     help="measure one part alone (for profiles); the line then holds that part only.  products / "
                          "gated-products: the sweep of the product kernels over rows and weight sizes; ceilings: "
                          "what the GPU itself reaches in reading HBM and in bfloat16 MFMA instructions")
@@ -471,7 +520,7 @@ def main():
                     help="decode steps run one at a time after the timed ones, for the p50 and p99 of a step's latency")
     ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="layer sizes: Gemma 2 2B (the default), 9B, 27B")
     ap.add_argument("--sizes", default="small,medium,large",
-                    help="--only zenuzen: which of the layer sizes small, medium, large (8 layers each, or --layers)")
+                    help="--only zenuzen / nemidra: which of the layer sizes small, medium, large (8 layers each, or --layers)")
     ap.add_argument("--requests", type=int, default=0,
                     help="instead of timed decode steps: a workload of this many requests through the scheduler")
     ap.add_argument("--prompt-min", type=int, default=128)
@@ -497,6 +546,9 @@ def main():
         return
     if args.only == "zenuzen":
         run_zenuzen(args)
+        return
+    if args.only == "nemidra":
+        run_nemidra(args)
         return
     d = dict(GEMMA2_2B, **SHAPES[args.shape])
     full_layers = d["num_hidden_layers"]
