@@ -483,6 +483,8 @@ def run_nemidra(args):
     for name in args.sizes.split(","):
         size = ZENUZEN_SIZES[name]
         for label, d in (("nemidra", nemidra_config(size, layers, positions)), ("zenuzen-equal-size", zenuzen_config(size, layers))):
+            if args.alone and label != "nemidra":
+                continue
             cfg = config_from_dict(d)
             model = random_model(cfg, 0, tdtype, torch.device("cuda:0"), std=0.02)
             pt, dt = run_executor_bench(model, size["vocab"], args.prefill_tokens, args.batch, args.context, args.steps,
@@ -521,6 +523,7 @@ def main():
     ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="layer sizes: Gemma 2 2B (the default), 9B, 27B")
     ap.add_argument("--sizes", default="small,medium,large",
                     help="--only zenuzen / nemidra: which of the layer sizes small, medium, large (8 layers each, or --layers)")
+    ap.add_argument("--alone", action="store_true", help="--only nemidra: without the closest model beside it (for profiles)")
     ap.add_argument("--requests", type=int, default=0,
                     help="instead of timed decode steps: a workload of this many requests through the scheduler")
     ap.add_argument("--prompt-min", type=int, default=128)

@@ -368,9 +368,6 @@ int sa_weighted_sum(const void* x, int64_t x_stride, float a, const void* y, int
                     void* out, int64_t out_stride, int T, int N, hipStream_t stream);
 
 // ---- matrix states that decay (linear_state.hip)
-// decay[t, c] = sigmoid(z)^(1 / tau), z = w2[c, :] . u[t, :] + b[c].
-int sa_gla_decay(const void* u, int u_dtype, int64_t u_stride, const void* w2, int w_dtype, const void* b, int b_dtype,
-                 float tau, int T, int R, int C, float* decay, hipStream_t stream);
 // raw [T, 2 H] (input gates, forget gates), bias [2 H] or null -> gates [T, 3 H]: decay, input factor, exp(-m), with
 // the running maximum m of every (slot, head) read from and left in m_state[slot * state_stride + h].
 int sa_exp_gates(const float* raw, int64_t raw_stride, const void* bias, int bias_dtype, float cap, int H,
@@ -378,10 +375,12 @@ int sa_exp_gates(const float* raw, int64_t raw_stride, const void* bias, int bia
                  hipStream_t stream);
 // S <- diag(a) S + c k v^T, out = S^T (q * q_mult) along every request's tokens; q, k, v are columns q_at, k_at, v_at
 // of proj's rows.  scalar: gates [T, >= 2 H] hold a and c per head; else gates [T, H dk] hold a per key channel and
-// c = 1.  ones: the state has a column dv whose value is always 1.  state [slot][H][dv + ones][dk]; out [T, H (dv + ones)].
+// c = 1; with tau > 0 these gates are z and a = sigmoid(z + gate_bias)^(1 / tau) (gate_bias [H dk] or null).  ones: the
+// state has a column dv whose value is always 1.  state [slot][H][dv + ones][dk]; out [T, H (dv + ones)].
 int sa_linear_state(const void* proj, int dtype, int64_t proj_stride, int q_at, int k_at, int v_at, float q_mult,
-                    const float* gates, int64_t gates_stride, int scalar, int H, int dk, int dv, int ones, float* state,
-                    int64_t state_stride, const int* seq_meta, int num_seqs, float* out, hipStream_t stream);
+                    const float* gates, int64_t gates_stride, const void* gate_bias, int bias_dtype, float tau, int scalar,
+                    int H, int dk, int dv, int ones, float* state, int64_t state_stride, const int* seq_meta, int num_seqs,
+                    float* out, hipStream_t stream);
 // x [T, H, size + 1] -> out[t, h, :] = unit_rms(x[t, h, :size] / (max(|x[t, h, size]|, floor[t, h]) + 1e-6)) * w[h, :]
 // * sigmoid(g[t, h, :]).
 int sa_normalized_readout(const float* x, const float* floor, int64_t floor_stride, const void* g, int g_dtype,

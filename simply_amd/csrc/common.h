@@ -105,6 +105,38 @@ __device__ __forceinline__ float lanes_sum(float v) {
   return v;
 }
 
+// The same for four values at once, step by step side by side: four chains of dependent steps that cover one another.
+// Every value's additions are those of lanes_sum, in its order.
+template <int LPC>
+__device__ __forceinline__ void lanes_sum4(float (&v)[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] += lane_exchange<0xB1>(v[i]);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] += lane_exchange<0x4E>(v[i]);
+  if (LPC >= 16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] += lane_exchange<0x141>(v[i]);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] += lane_exchange<0x140>(v[i]);
+  }
+  if (LPC >= 32) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned u = __float_as_uint(v[i]);
+      const auto rows = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+      v[i] = __uint_as_float(rows[0]) + __uint_as_float(rows[1]);
+    }
+  }
+  if (LPC == 64) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned u = __float_as_uint(v[i]);
+      const auto halves = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+      v[i] = __uint_as_float(halves[0]) + __uint_as_float(halves[1]);
+    }
+  }
+}
+
 // Sum over a block of up to 1024 threads; every thread gets the result.  The
 // order of additions depends only on the block size, never on the data.
 __device__ inline float block_sum(float v, float* scratch /* >= 16 floats */) {

@@ -6,9 +6,9 @@
 // (the matrix memory with exponential gates, whose decay and factor come from a running maximum of the logarithms
 // of its gates; its normalizer n_t = a_t n_(t-1) + c_t k_t is one more column of S whose value is always 1).
 //
-//   gla_decay_kernel          a = sigmoid(z)^(1/tau), z = W2 u + b, from the low-rank projection u
 //   exp_gates_kernel          i, f from their projections, the running maximum m, a = exp(f + m' - m), c = exp(i - m)
-//   linear_state_kernel       the recurrence, prefill and decode
+//   linear_state_kernel       the recurrence, prefill and decode; a decay per channel may come as z with
+//                             a = sigmoid(z + b)^(1/tau), computed as the tile is staged
 //   normalized_readout_kernel o / (max(|n.q|, exp(-m)) + 1e-6), each head to unit RMS, times a weight and sigmoid(gate)
 //
 // A request's tokens of this step are rows first .. first + count - 1 (seq_meta [S, 4]: state slot, first row, count,
@@ -21,20 +21,6 @@
 namespace sa {
 
 __device__ inline float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
-
-// decay[t, c] = exp(log_sigmoid(z) / tau), z = sum_r w2[c, r] u[t, r] + b[c].  A thread per (token, channel).
-__global__ __launch_bounds__(256) void gla_decay_kernel(const void* __restrict__ u, int u_dtype, int64_t u_stride,
-                                                        const void* __restrict__ w2, int w_dtype,
-                                                        const void* __restrict__ b, int b_dtype, float inv_tau, int R,
-                                                        int C, float* __restrict__ decay) {
-  const int t = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= C) return;
-  float z = 0.f;
-  for (int r = 0; r < R; ++r)
-    z = fmaf(load_f(w2, w_dtype, static_cast<size_t>(c) * R + r), load_f(u, u_dtype, static_cast<size_t>(t) * u_stride + r), z);
-  if (b != nullptr) z += load_f(b, b_dtype, c);
-  decay[static_cast<size_t>(t) * C + c] = expf(log_sigmoid(z) * inv_tau);
-}
 
 // The gates of the matrix memory.  raw [T, 2 H]: the projections of the input and forget gates (input gates first),
 // bias [2 H] alike (null: none).  i = cap tanh((x_i + b_i) / cap), f = log_sigmoid(cap tanh((x_f + b_f) / cap));
@@ -92,8 +78,9 @@ constexpr int kStateTokens = 16;
 template <int DK, int LPC, bool SCALAR, typename XT>
 __global__ __launch_bounds__(256) void linear_state_kernel(
     const XT* __restrict__ proj, int64_t proj_stride, int q_at, int k_at, int v_at, float q_mult,
-    const float* __restrict__ gates, int64_t gates_stride, int H, int dk, int dv, int ones, float* __restrict__ state,
-    int64_t state_stride, const int* __restrict__ seq_meta, float* __restrict__ out) {
+    const float* __restrict__ gates, int64_t gates_stride, const void* __restrict__ gate_bias, int bias_dtype,
+    float inv_tau, int H, int dk, int dv, int ones, float* __restrict__ state, int64_t state_stride,
+    const int* __restrict__ seq_meta, float* __restrict__ out) {
   constexpr int R = DK / LPC, COLS = 256 / LPC;
   constexpr int AD = SCALAR ? 1 : DK;
   __shared__ float qs[kStateTokens][DK], ks[kStateTokens][DK], vs[kStateTokens][COLS], as[kStateTokens][AD],
@@ -123,7 +110,15 @@ __global__ __launch_bounds__(256) void linear_state_kernel(
       const XT* row = proj + t * proj_stride;
       pq[i] = ok ? to_float(row[q_at + h * dk + d]) * q_mult : 0.f;
       pk[i] = ok ? to_float(row[k_at + h * dk + d]) : 0.f;
-      if constexpr (!SCALAR) pa[i] = ok ? gates[t * gates_stride + h * dk + d] : 0.f;
+      if constexpr (!SCALAR) {
+        // inv_tau > 0: the gates are z, and the decay is sigmoid(z + bias)^(1 / tau)
+        float a = ok ? gates[t * gates_stride + h * dk + d] : 0.f;
+        if (ok && inv_tau > 0.f) {
+          if (gate_bias != nullptr) a += load_f(gate_bias, bias_dtype, h * dk + d);
+          a = expf(log_sigmoid(a) * inv_tau);
+        }
+        pa[i] = a;
+      }
     }
 #pragma unroll
     for (int i = 0; i < PV; ++i) {
@@ -152,48 +147,36 @@ __global__ __launch_bounds__(256) void linear_state_kernel(
     if constexpr (SCALAR) if (tid < 2 * kStateTokens) cs[tid / 2][tid % 2] = pc;
     __syncthreads();
     if (t0 + kStateTokens < count) fetch(t0 + kStateTokens);
-    struct Operands {
-      float k[R], q[R], a[SCALAR ? 1 : R], v, c;
-    };
-    auto read = [&](Operands& x, int j) __attribute__((always_inline)) {
+    // four tokens at a time: their updates follow one another, their sums across the lanes run side by side (a wave
+    // issues in order, and one such sum alone is a chain of dependent steps that nothing else covers)
+    for (int j0 = 0; j0 < tn; j0 += 4) {
+      float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        x.k[r] = ks[j][r * LPC + part];
-        x.q[r] = qs[j][r * LPC + part];
-        if constexpr (!SCALAR) x.a[r] = as[j][(r * LPC + part) % AD];
-      }
-      x.v = vs[j][tid / LPC];
-      if constexpr (SCALAR) {
-        x.a[0] = cs[j][0];
-        x.c = cs[j][1];
-      } else {
-        x.c = 1.f;
-      }
-    };
-    auto token = [&](const Operands& x, int j) __attribute__((always_inline)) {
-      const float u = SCALAR ? x.c * x.v : x.v;
-      float d[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int i = 0; i < 4; ++i) {
+        const int j = j0 + i;
+        if (j < tn) {   // (uniform)
+          float u = vs[j][tid / LPC], a0 = 1.f;
+          if constexpr (SCALAR) {
+            a0 = cs[j][0];
+            u *= cs[j][1];
+          }
+          float d[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        float a;
-        if constexpr (SCALAR) a = x.a[0];
-        else a = x.a[r];
-        s[r] = fmaf(x.k[r], u, s[r] * a);
-        d[r % 4] = fmaf(s[r], x.q[r], d[r % 4]);
+          for (int r = 0; r < R; ++r) {
+            float a = a0;
+            if constexpr (!SCALAR) a = as[j][(r * LPC + part) % AD];
+            s[r] = fmaf(ks[j][r * LPC + part], u, s[r] * a);
+            d[r % 4] = fmaf(s[r], qs[j][r * LPC + part], d[r % 4]);
+          }
+          o[i] = (d[0] + d[1]) + (d[2] + d[3]);
+        }
       }
-      float o = (d[0] + d[1]) + (d[2] + d[3]);
-      o = lanes_sum<LPC>(o);
-      if (live && part == 0)
-        out[static_cast<size_t>(first + t0 + j) * (static_cast<size_t>(H) * CT) + static_cast<size_t>(h) * CT + col] = o;
-    };
-    Operands A, B;
-    read(A, 0);
-    for (int j = 0; j < tn; j += 2) {
-      if (j + 1 < tn) read(B, j + 1);
-      token(A, j);
-      if (j + 1 < tn) {
-        if (j + 2 < tn) read(A, j + 2);
-        token(B, j + 1);
+      lanes_sum4<LPC>(o);
+      if (live && part == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (j0 + i < tn)
+            out[static_cast<size_t>(first + t0 + j0 + i) * (static_cast<size_t>(H) * CT) + static_cast<size_t>(h) * CT + col] = o[i];
       }
     }
   }
@@ -233,22 +216,6 @@ __global__ __launch_bounds__(kWave) void normalized_readout_kernel(
 
 using namespace sa;
 
-extern "C" int sa_gla_decay(const void* u, int u_dtype, int64_t u_stride, const void* w2, int w_dtype, const void* b,
-                            int b_dtype, float tau, int T, int R, int C, float* decay, hipStream_t stream) {
-  if (T == 0) return 0;
-  SA_REQUIRE(T > 0 && R > 0 && C > 0 && u_stride >= R && tau > 0.f, "gla_decay: bad sizes T=%d R=%d C=%d tau=%g", T, R, C,
-             static_cast<double>(tau));
-  SA_REQUIRE(u != nullptr && w2 != nullptr && decay != nullptr, "gla_decay: a null pointer");
-  SA_REQUIRE(T <= 65535 * 1024, "gla_decay: too many tokens");
-  for (int t0 = 0; t0 < T; t0 += 65535) {
-    const int rows = T - t0 < 65535 ? T - t0 : 65535;
-    const char* ub = static_cast<const char*>(u) + static_cast<size_t>(t0) * u_stride * (u_dtype == kF32 ? 4 : 2);
-    gla_decay_kernel<<<dim3((C + 255) / 256, rows), 256, 0, stream>>>(ub, u_dtype, u_stride, w2, w_dtype, b, b_dtype,
-                                                                     1.f / tau, R, C, decay + static_cast<size_t>(t0) * C);
-  }
-  return check_launch("gla_decay");
-}
-
 extern "C" int sa_exp_gates(const float* raw, int64_t raw_stride, const void* bias, int bias_dtype, float cap, int H,
                             float* m_state, int64_t state_stride, const int* seq_meta, int num_seqs, float* gates,
                             hipStream_t stream) {
@@ -263,9 +230,9 @@ extern "C" int sa_exp_gates(const float* raw, int64_t raw_stride, const void* bi
 }
 
 extern "C" int sa_linear_state(const void* proj, int dtype, int64_t proj_stride, int q_at, int k_at, int v_at,
-                               float q_mult, const float* gates, int64_t gates_stride, int scalar, int H, int dk, int dv,
-                               int ones, float* state, int64_t state_stride, const int* seq_meta, int num_seqs,
-                               float* out, hipStream_t stream) {
+                               float q_mult, const float* gates, int64_t gates_stride, const void* gate_bias,
+                               int bias_dtype, float tau, int scalar, int H, int dk, int dv, int ones, float* state,
+                               int64_t state_stride, const int* seq_meta, int num_seqs, float* out, hipStream_t stream) {
   if (num_seqs == 0) return 0;
   SA_REQUIRE(num_seqs > 0 && num_seqs <= 65535 && H > 0 && H <= 65535 && dk > 0 && dv > 0 && (ones == 0 || ones == 1),
              "linear_state: bad sizes S=%d H=%d dk=%d dv=%d", num_seqs, H, dk, dv);
@@ -280,10 +247,12 @@ extern "C" int sa_linear_state(const void* proj, int dtype, int64_t proj_stride,
              "linear_state: a null pointer");
   SA_REQUIRE(dtype == kF32 || dtype == kBF16, "linear_state: unknown dtype %d", dtype);
   SA_REQUIRE(CT <= 65535 * 4, "linear_state: too many columns");
+  SA_REQUIRE(tau >= 0.f && (scalar == 0 || tau == 0.f), "linear_state: tau belongs to decays per channel and is not negative");
+  const float inv_tau = tau > 0.f ? 1.f / tau : 0.f;
 #define SA_STATE_LAUNCH(DK, LPC, SC, XT)                                                                             \
   linear_state_kernel<DK, LPC, SC, XT><<<dim3(num_seqs, H, (CT + 256 / LPC - 1) / (256 / LPC)), 256, 0, stream>>>(   \
-      static_cast<const XT*>(proj), proj_stride, q_at, k_at, v_at, q_mult, gates, gates_stride, H, dk, dv, ones, state, \
-      state_stride, seq_meta, out)
+      static_cast<const XT*>(proj), proj_stride, q_at, k_at, v_at, q_mult, gates, gates_stride, gate_bias, bias_dtype, \
+      inv_tau, H, dk, dv, ones, state, state_stride, seq_meta, out)
 #define SA_STATE_SIZES(SC, XT)                       \
   do {                                               \
     if (dk <= 16) SA_STATE_LAUNCH(16, 4, SC, XT);    \

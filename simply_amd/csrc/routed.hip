@@ -208,6 +208,118 @@ __global__ __launch_bounds__(256) void expert_product_kernel(
   }
 }
 
+// The same products for tiles of 64 rows (steps that bring an expert many rows), bfloat16: a workgroup takes the tile's
+// rows and 128 columns, a wave 32 of them (two column tiles) for all four sub-tiles of 16 rows.  The rows' operands of
+// 64 columns of K at a time go through LDS in operand order (every wave needs all of them: read from memory once
+// instead of four times), asked for a chunk ahead into registers; the weights' operands come straight from their
+// tiles.  A row's sums are those of the kernel above, in its order.
+constexpr int kChunkK = 64;
+template <bool GATED>
+__global__ __launch_bounds__(256) void expert_product_rows64_kernel(
+    const bf16* __restrict__ a, int64_t a_stride, int a_by_token, int top, const bf16* __restrict__ w1,
+    const bf16* __restrict__ w2, int N, int K, const int* __restrict__ sorted, const int* __restrict__ plan, int act,
+    void* __restrict__ out, int64_t out_stride, int out_by_pair) {
+  __shared__ bf16x8 rows_lds[4][kChunkK / 32][kWave];   // [sub-tile of 16 rows][k tile of the chunk][lane]
+  __shared__ int pair_of[kTileRowsMax];
+  const int tile = blockIdx.x;
+  if (tile >= plan[0]) return;
+  const int e = plan[1 + 2 * tile], packed = plan[2 + 2 * tile];
+  const int row0 = packed / 128, rows = packed % 128;
+  const int tid = threadIdx.x, wave = tid / kWave, lane = tid % kWave;
+  const int r = lane % 16, kq = lane / 16;
+  const int n0 = (blockIdx.y * 4 + wave) * 32;
+  const bool mine = n0 < N;   // (a wave without columns still stages rows and meets the barriers)
+  if (tid < kTileRowsMax) pair_of[tid] = sorted[row0 + (tid < rows ? tid : rows - 1)];
+  __syncthreads();
+  const bool aligned = a_stride % 8 == 0;
+  // staging: this thread's two pieces of 8 elements of a chunk, and where they go
+  const bf16* src[2];
+  int koff[2];
+  bf16x8* dst[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int combo = wave + 4 * i, sub = combo / 2, kt = combo % 2;
+    const int row = sub * 16 + r, rr = row < rows ? row : rows - 1;
+    src[i] = a + static_cast<size_t>(a_by_token ? pair_of[rr] / top : row0 + rr) * a_stride;
+    koff[i] = kt * 32 + kq * 8;
+    dst[i] = &rows_lds[sub][kt][lane];
+  }
+  bf16x8 staged[2];
+  auto fetch = [&](int c) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int k = c * kChunkK + koff[i];
+      if (aligned && k + 8 <= K) {
+        staged[i] = load8(src[i] + k);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          staged[i][j] = k + j < K ? __builtin_bit_cast(__bf16, src[i][k + j]) : static_cast<__bf16>(0.f);
+      }
+    }
+  };
+  const int Nt = (N + 15) / 16, Kt = (K + 31) / 32;
+  const int nsub = (rows + 15) / 16;
+  floatx4 accg[4][2], accu[4][2];
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) accg[s][j] = accu[s][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const int chunks = (K + kChunkK - 1) / kChunkK;
+  fetch(0);
+  for (int c = 0; c < chunks; ++c) {
+    __syncthreads();   // the chunk before has been read
+    *dst[0] = staged[0];
+    *dst[1] = staged[1];
+    __syncthreads();
+    if (c + 1 < chunks) fetch(c + 1);
+    if (!mine) continue;
+#pragma unroll
+    for (int kt = 0; kt < kChunkK / 32; ++kt) {
+      const int ktg = c * (kChunkK / 32) + kt;
+      if (ktg >= Kt) break;
+      bf16x8 gv[2], uv[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int nt = n0 / 16 + j < Nt ? n0 / 16 + j : Nt - 1;
+        const size_t at = ((static_cast<size_t>(e) * Nt + nt) * Kt + ktg) * 512 + lane * 8;
+        gv[j] = load8(w1 + at);
+        if constexpr (GATED) uv[j] = load8(w2 + at);
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        if (s >= nsub) break;
+        const bf16x8 av = rows_lds[s][kt][lane];
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          accg[s][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gv[j], av, accg[s][j], 0, 0, 0);
+          if constexpr (GATED) accu[s][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uv[j], av, accu[s][j], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if (!mine) return;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const int row = s * 16 + r;
+    if (row >= rows) continue;
+    const size_t orow = static_cast<size_t>(out_by_pair ? pair_of[row] : row0 + row) * out_stride;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + j * 16 + kq * 4 + i;
+        if (n >= N) continue;
+        if constexpr (GATED) {
+          const float v = gated_activation(act, to_float(float_to_bf16(accg[s][j][i]))) * to_float(float_to_bf16(accu[s][j][i]));
+          static_cast<bf16*>(out)[orow + n] = float_to_bf16(v);
+        } else {
+          static_cast<float*>(out)[orow + n] = accg[s][j][i];
+        }
+      }
+  }
+}
+
 // out[t, d] = sum_k weights[t, k] * y[t * top + k, d] (in the order of k) + sigmoid(gate[t]) * shared[t, d].
 __global__ void combine_kernel(const float* __restrict__ y, const float* __restrict__ weights, int top,
                                const void* __restrict__ shared, int shared_dtype, int64_t shared_stride,
@@ -280,8 +392,15 @@ extern "C" int sa_expert_product(const void* a, int dtype, int64_t a_stride, int
       if (gated) SA_EXPERT(bf16, true, 1);
       else SA_EXPERT(bf16, false, 1);
     } else {
-      if (gated) SA_EXPERT(bf16, true, 4);
-      else SA_EXPERT(bf16, false, 4);
+      const dim3 wide(grid.x, (N + 127) / 128);
+      if (gated)
+        expert_product_rows64_kernel<true><<<wide, 256, 0, stream>>>(
+            static_cast<const bf16*>(a), a_stride, a_by_token, top, static_cast<const bf16*>(w1),
+            static_cast<const bf16*>(w2), N, K, sorted, plan, act, out, out_stride, out_by_pair);
+      else
+        expert_product_rows64_kernel<false><<<wide, 256, 0, stream>>>(
+            static_cast<const bf16*>(a), a_stride, a_by_token, top, static_cast<const bf16*>(w1), nullptr, N, K, sorted,
+            plan, act, out, out_stride, out_by_pair);
     }
   } else {
     if (gated) SA_EXPERT(float, true, 1);

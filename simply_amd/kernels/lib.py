@@ -73,9 +73,8 @@ _SIGNATURES = {
     "sa_token_gate": [_P, _I, _L, _P, _P, _I, _L, _I, _I, _I, _I, _P],
     "sa_bias_add": [_P, _I, _L, _P, _I, _I, _I, _P],
     "sa_weighted_sum": [_P, _L, _F, _P, _L, _F, _I, _P, _L, _I, _I, _P],
-    "sa_gla_decay": [_P, _I, _L, _P, _I, _P, _I, _F, _I, _I, _I, _P, _P],
     "sa_exp_gates": [_P, _L, _P, _I, _F, _I, _P, _L, _P, _I, _P, _P],
-    "sa_linear_state": [_P, _I, _L, _I, _I, _I, _F, _P, _L, _I, _I, _I, _I, _I, _P, _L, _P, _I, _P, _P],
+    "sa_linear_state": [_P, _I, _L, _I, _I, _I, _F, _P, _L, _P, _I, _F, _I, _I, _I, _I, _I, _P, _L, _P, _I, _P, _P],
     "sa_normalized_readout": [_P, _P, _L, _P, _I, _L, _P, _I, _F, _P, _I, _L, _I, _I, _I, _P],
     "sa_route": [_P, _L, _I, _I, _I, _F, _P, _P, _P],
     "sa_expert_sort": [_P, _I, _I, _I, _P, _P, _I, _P],

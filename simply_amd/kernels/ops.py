@@ -1124,21 +1124,6 @@ def weighted_sum(x: torch.Tensor, a: float, y: torch.Tensor, b: float, out: torc
 
 # --------------------------------------------------------------------------- matrix states that decay
 
-def gla_decay(u: torch.Tensor, w2: torch.Tensor, bias: torch.Tensor | None, tau: float) -> torch.Tensor:
-    """float32 [T, C]: sigmoid(u . w2^T + bias)^(1 / tau).  u [T, R] (rows of a projection), w2 [C, R] row-major."""
-    _dev(u, w2, bias)
-    T, R = u.shape
-    if w2.dim() != 2 or w2.shape[1] != R or not w2.is_contiguous():
-        raise KernelError(f"gla_decay: the second factor {tuple(w2.shape)} does not go with rows of {R}")
-    C = w2.shape[0]
-    if bias is not None and (bias.numel() != C or not bias.is_contiguous()):
-        raise KernelError("gla_decay: one bias per channel")
-    out = torch.empty((T, C), dtype=torch.float32, device=u.device)
-    _lib.call("sa_gla_decay", _ptr(u), _code(u), _rows(u, "gla_decay: u"), _ptr(w2), _code(w2), _ptr(bias),
-              _code(bias) if bias is not None else 0, float(tau), T, R, C, _ptr(out), _stream())
-    return out
-
-
 def exp_gates(raw: torch.Tensor, bias: torch.Tensor | None, cap: float, num_heads: int, m_state: torch.Tensor,
               seq_meta: torch.Tensor, num_seqs: int) -> torch.Tensor:
     """The gates of a matrix memory with exponential gates.  raw float32 [T, 2 H] (input gates' projections, then forget
@@ -1161,10 +1146,11 @@ def exp_gates(raw: torch.Tensor, bias: torch.Tensor | None, cap: float, num_head
 
 def linear_state(proj: torch.Tensor, q_at: int, k_at: int, v_at: int, q_mult: float, gates: torch.Tensor, scalar: bool,
                  num_heads: int, key_dim: int, value_dim: int, ones: bool, state: torch.Tensor, seq_meta: torch.Tensor,
-                 num_seqs: int) -> torch.Tensor:
+                 num_seqs: int, *, decay_bias: torch.Tensor | None = None, tau: float | None = None) -> torch.Tensor:
     """S <- diag(a) S + c k v^T, o = S^T (q * q_mult) along each request's tokens, from and into state float32 [slots,
     >= H * dk * (dv + ones)] (per head [dv + ones][dk]).  q, k, v: columns q_at, k_at, v_at of proj's rows, H heads
-    each.  scalar: gates float32 [T, >= 2 H] hold a and c per head; else [T, H * dk] hold a per key channel, c = 1.
+    each.  scalar: gates float32 [T, >= 2 H] hold a and c per head; else [T, H * dk] hold a per key channel, c = 1;
+    with `tau` these hold z instead, and a = sigmoid(z + decay_bias)^(1 / tau) (decay_bias [H * dk] or None).
     ones: one more column whose value is always 1 (a normalizer).  Returns float32 [T, H * (dv + ones)]."""
     _dev(proj, gates, state, seq_meta)
     T = proj.shape[0]
@@ -1174,9 +1160,15 @@ def linear_state(proj: torch.Tensor, q_at: int, k_at: int, v_at: int, q_mult: fl
     if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < H * dk * CT:
         raise KernelError("linear_state: the state must be float32 [slots, >= H * dk * (dv + ones)]")
     _seq_meta(seq_meta, num_seqs, "linear_state")
+    if (tau is not None or decay_bias is not None) and (scalar or tau is None or tau <= 0):
+        raise KernelError("linear_state: tau (positive) and a bias belong to decays per channel")
+    if decay_bias is not None and (decay_bias.numel() != H * dk or not decay_bias.is_contiguous()):
+        raise KernelError("linear_state: one bias per key channel")
+    _dev(decay_bias)
     out = torch.empty((T, H * CT), dtype=torch.float32, device=proj.device)
     _lib.call("sa_linear_state", _ptr(proj), _code(proj), _rows(proj, "linear_state: proj"), int(q_at), int(k_at), int(v_at),
-              float(q_mult), _ptr(gates), _rows(gates, "linear_state: gates"), int(bool(scalar)), H, dk, dv,
+              float(q_mult), _ptr(gates), _rows(gates, "linear_state: gates"), _ptr(decay_bias),
+              _code(decay_bias) if decay_bias is not None else 0, float(tau or 0.0), int(bool(scalar)), H, dk, dv,
               int(bool(ones)), _ptr(state), state.stride(0), _ptr(seq_meta), int(num_seqs), _ptr(out), _stream())
     return out
 

@@ -44,7 +44,7 @@ class GatedLinearAttention(Mixer):
         D, H, dk, dv, R = self.hidden_size, self.num_heads, self.key_dim, self.value_dim, self.decay_rank
         return {"q_proj": ParamSpec((H * dk, D)), "k_proj": ParamSpec((H * dk, D)), "v_proj": ParamSpec((H * dv, D)),
                 "gate_proj": ParamSpec((H * dv, D)), "o_proj": ParamSpec((D, H * dv)),
-                "decay_in": ParamSpec((R, D)), "decay_out": ParamSpec((H * dk, R), role="vector"),
+                "decay_in": ParamSpec((R, D)), "decay_out": ParamSpec((H * dk, R)),
                 "decay_bias": ParamSpec((H * dk,), role="vector", init="norm"),
                 "norm": ParamSpec((dv,), role="vector", init="norm")}
 
@@ -54,7 +54,7 @@ class GatedLinearAttention(Mixer):
         self.in_proj = as_product_weight(torch.cat([t["q_proj"], t["k_proj"], t["v_proj"], t["gate_proj"],
                                                     t["decay_in"]], dim=0).contiguous())
         self.o_proj = as_product_weight(t["o_proj"])
-        self.decay_out, self.decay_bias = t["decay_out"].contiguous(), t["decay_bias"].contiguous()
+        self.decay_out, self.decay_bias = as_product_weight(t["decay_out"]), t["decay_bias"].contiguous()
         self.norm = t["norm"].contiguous()
 
     def cache_need(self):
@@ -68,9 +68,11 @@ class GatedLinearAttention(Mixer):
         g_at = 2 * C + H * dv
         u_at = g_at + H * dv
         proj = project(x, self.in_proj)
-        decay = ops.gla_decay(proj[:, u_at:u_at + R], self.decay_out, self.decay_bias, self.tau)
-        o = ops.linear_state(proj, 0, C, 2 * C, dk ** -0.5, decay, False, H, dk, dv, False, cache.state, ctx.seq_meta,
-                             ctx.num_seqs)
+        # the decay's second factor is a product of its own, kept in 32-bit; sigmoid(. + bias)^(1 / tau) is computed
+        # where the recurrence stages its tiles
+        z = ops.gemm(proj[:, u_at:u_at + R], self.decay_out, out_dtype=torch.float32)
+        o = ops.linear_state(proj, 0, C, 2 * C, dk ** -0.5, z, False, H, dk, dv, False, cache.state, ctx.seq_meta,
+                             ctx.num_seqs, decay_bias=self.decay_bias, tau=self.tau)
         z = ops.gated_heads(o, proj[:, g_at:g_at + H * dv], H, dv, kind=ops.GATE_SILU, weight=self.norm,
                             eps=self.norm_eps, out_dtype=ctx.dtype)
         return ops.gemm(z, self.o_proj)

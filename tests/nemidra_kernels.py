@@ -54,15 +54,16 @@ def matrix_states(ops, dev, dtype, sizes=((3, 48, 32), (2, 32, 48), (2, 128, 64)
         m, T = _meta([1, 3, 40, 17], [1, 3, 0, 2], [9, 0, 4, 30])
         C = H * dk
         proj = (torch.randn(T, 2 * C + 2 * H * dv + 8, generator=g) * 0.5).to(dtype)
-        w2, bias = torch.randn(C, 8, generator=g).to(dtype), torch.randn(C, generator=g).to(dtype)
-        decay = ref.gla_decay(proj[:, -8:], w2, bias, 4.0)
-        _cmp(ops.gla_decay(proj.to(dev)[:, -8:], w2.to(dev), bias.to(dev), 4.0), decay, 1e-5, ("gla_decay", H, dk))
-        st = torch.randn(4, C * dv + 5, generator=g) * 0.3
-        st_d = st.clone().to(dev)
-        got = ops.linear_state(proj.to(dev), 0, C, 2 * C, dk ** -0.5, decay.to(dev), False, H, dk, dv, False, st_d, m.to(dev), 4)
-        want = ref.linear_state(proj, 0, C, 2 * C, dk ** -0.5, decay, False, H, dk, dv, False, st, m, 4)
-        _cmp(got, want, 3e-5, ("linear_state, decays per channel", H, dk, dv))
-        _cmp(st_d, st, 3e-5, "its state")
+        z, bias = torch.randn(T, C, generator=g) * 2, torch.randn(C, generator=g).to(dtype)
+        for kw, kw_d in (({}, {}), (dict(decay_bias=bias, tau=4.0), dict(decay_bias=bias.to(dev), tau=4.0))):
+            gates = z if kw else torch.sigmoid(z)    # z with a bias and tau, or decays as they are
+            st = torch.randn(4, C * dv + 5, generator=g) * 0.3
+            st_d = st.clone().to(dev)
+            got = ops.linear_state(proj.to(dev), 0, C, 2 * C, dk ** -0.5, gates.to(dev), False, H, dk, dv, False, st_d,
+                                   m.to(dev), 4, **kw_d)
+            want = ref.linear_state(proj, 0, C, 2 * C, dk ** -0.5, gates, False, H, dk, dv, False, st, m, 4, **kw)
+            _cmp(got, want, 3e-5, ("linear_state, decays per channel", H, dk, dv, bool(kw)))
+            _cmp(st_d, st, 3e-5, "its state")
         raw, gb = torch.randn(T, 2 * H, generator=g) * 3, torch.randn(2 * H, generator=g).to(dtype)
         words = C * (dv + 1)
         st = torch.randn(4, words + H, generator=g) * 0.3

@@ -519,13 +519,6 @@ def weighted_sum(x, a, y, b, out=None):
 
 # --------------------------------------------------------------------------- matrix states that decay
 
-def gla_decay(u, w2, bias, tau):
-    z = _f(u) @ _f(w2).T
-    if bias is not None:
-        z = z + _f(bias)
-    return torch.exp(torch.nn.functional.logsigmoid(z) / tau).to(torch.float32)
-
-
 def exp_gates(raw, bias, cap, num_heads, m_state, seq_meta, num_seqs):
     H = num_heads
     x = _f(raw) + (_f(bias) if bias is not None else 0.0)
@@ -544,8 +537,11 @@ def exp_gates(raw, bias, cap, num_heads, m_state, seq_meta, num_seqs):
 
 
 def linear_state(proj, q_at, k_at, v_at, q_mult, gates, scalar, num_heads, key_dim, value_dim, ones, state, seq_meta,
-                 num_seqs):
+                 num_seqs, *, decay_bias=None, tau=None):
     H, dk, dv = num_heads, key_dim, value_dim
+    if tau is not None:   # the gates are z: a = sigmoid(z + bias)^(1 / tau)
+        z = _f(gates) + (_f(decay_bias) if decay_bias is not None else 0.0)
+        gates = torch.exp(torch.nn.functional.logsigmoid(z) / tau)
     CT = dv + int(bool(ones))
     T = proj.shape[0]
     p, g = _f(proj), _f(gates)
