@@ -361,12 +361,6 @@ int sa_embed_sum(const int* tokens, const int* positions, const int* seq_meta, i
 // z[t, j] = act(z[t, j]) * table[tokens[t], col0 + j], in place.
 int sa_token_gate(void* z, int dtype, int64_t stride, const int* tokens, const void* table, int table_dtype,
                   int64_t table_stride, int col0, int T, int N, int act, hipStream_t stream);
-// For steps of few tokens, in one launch: x = h[t] in the tables' type; g = act(wg x) * table[tokens[t], col0 ..];
-// y = wpt^T g; h[t] += y / sqrt(mean(y^2) + eps) * w.  wg [dim, D] and wpt [dim, D] row-major, of the table's type.
-int sa_token_side_few_takes(int T, int D, int dim);
-int sa_token_side_few(float* h, const int* tokens, const void* table, int dtype, int64_t table_stride, int col0,
-                      const void* wg, const void* wpt, const void* w, int w_dtype, float eps, int act, int T, int D, int dim,
-                      hipStream_t stream);
 // x[t, n] += b[n], in place.
 int sa_bias_add(void* x, int dtype, int64_t stride, const void* b, int b_dtype, int T, int N, hipStream_t stream);
 // out = a x + b y.

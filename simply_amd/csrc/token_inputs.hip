@@ -52,50 +52,6 @@ __global__ void token_gate_kernel(void* __restrict__ z, int dtype, int64_t strid
   store_f(z, dtype, at, gated_activation_exact(act, load_f(z, dtype, at)) * e);
 }
 
-// The whole per-layer token input for a step of few tokens, one workgroup a token:
-//   x = h[t] (rounded to T);  z = Wg x;  g = act(z) * e[token];  y = Wp g;  h[t] += y / sqrt(mean(y^2) + eps) * w.
-// wg [dim, D] and wpt [dim, D] (the projection transposed) are row-major, so that both products read whole rows.
-// z, g and y are rounded to T where the separate kernels store them in T.
-constexpr int kSideDimMax = 256;
-template <typename T>
-__global__ __launch_bounds__(256) void token_side_few_kernel(float* __restrict__ h, const int* __restrict__ tokens,
-                                                             const T* __restrict__ table, int64_t table_stride, int col0,
-                                                             const T* __restrict__ wg, const T* __restrict__ wpt,
-                                                             const void* __restrict__ w, int w_dtype, float eps, int act,
-                                                             int D, int dim) {
-  extern __shared__ float x[];   // [D]
-  __shared__ float g[kSideDimMax];
-  __shared__ float scratch[16];
-  const int t = blockIdx.x, tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  float* row = h + static_cast<size_t>(t) * D;
-  for (int d = tid; d < D; d += 256) x[d] = to_float(from_float<T>(row[d]));
-  __syncthreads();
-  const T* e = table + static_cast<size_t>(tokens[t]) * table_stride + col0;
-  for (int j = wave; j < dim; j += 4) {
-    const T* wr = wg + static_cast<size_t>(j) * D;
-    float acc = 0.f;
-    for (int d = lane; d < D; d += kWave) acc = fmaf(to_float(wr[d]), x[d], acc);
-    acc = wave_sum(acc);
-    if (lane == 0) {
-      const float z = to_float(from_float<T>(acc));
-      g[j] = to_float(from_float<T>(gated_activation_exact(act, z) * to_float(e[j])));
-    }
-  }
-  __syncthreads();
-  // y[d] for this thread's d = tid, tid + 256, ...: kept in x's place
-  float ss = 0.f;
-  for (int d = tid; d < D; d += 256) {
-    float acc = 0.f;
-    for (int j = 0; j < dim; ++j) acc = fmaf(to_float(wpt[static_cast<size_t>(j) * D + d]), g[j], acc);
-    acc = to_float(from_float<T>(acc));
-    x[d] = acc;
-    ss = fmaf(acc, acc, ss);
-  }
-  ss = block_sum(ss, scratch);
-  const float r = 1.f / sqrtf(ss / static_cast<float>(D) + eps);
-  for (int d = tid; d < D; d += 256) row[d] += x[d] * r * load_f(w, w_dtype, d);
-}
-
 // x[t, n] += b[n] in place.
 __global__ void bias_add_kernel(void* __restrict__ x, int dtype, int64_t stride, const void* __restrict__ b, int b_dtype,
                                 int N) {
@@ -149,34 +105,6 @@ extern "C" int sa_token_gate(void* z, int dtype, int64_t stride, const int* toke
   token_gate_kernel<<<dim3((N + 255) / 256, T), 256, 0, stream>>>(z, dtype, stride, tokens, table, table_dtype,
                                                                   table_stride, col0, N, act);
   return check_launch("token_gate");
-}
-
-extern "C" int sa_token_side_few_takes(int T, int D, int dim) {
-  return T >= 1 && T <= 16 && dim >= 1 && dim <= kSideDimMax && D >= 1 && D <= 12288;
-}
-
-extern "C" int sa_token_side_few(float* h, const int* tokens, const void* table, int dtype, int64_t table_stride, int col0,
-                                 const void* wg, const void* wpt, const void* w, int w_dtype, float eps, int act, int T,
-                                 int D, int dim, hipStream_t stream) {
-  if (T == 0) return 0;
-  SA_REQUIRE(sa_token_side_few_takes(T, D, dim), "token_side_few: at most 16 tokens, %d table columns and a width of 12288",
-             kSideDimMax);
-  SA_REQUIRE(h != nullptr && tokens != nullptr && table != nullptr && wg != nullptr && wpt != nullptr && w != nullptr,
-             "token_side_few: a null pointer");
-  SA_REQUIRE(col0 >= 0 && table_stride >= col0 + dim && eps >= 0.f, "token_side_few: bad columns or eps");
-  SA_REQUIRE(act >= 0 && act < kNumActivations, "token_side_few: unknown activation %d", act);
-  const size_t lds = static_cast<size_t>(D) * sizeof(float);
-  if (dtype == kBF16)
-    token_side_few_kernel<bf16><<<T, 256, lds, stream>>>(h, tokens, static_cast<const bf16*>(table), table_stride, col0,
-                                                         static_cast<const bf16*>(wg), static_cast<const bf16*>(wpt), w,
-                                                         w_dtype, eps, act, D, dim);
-  else if (dtype == kF32)
-    token_side_few_kernel<float><<<T, 256, lds, stream>>>(h, tokens, static_cast<const float*>(table), table_stride, col0,
-                                                          static_cast<const float*>(wg), static_cast<const float*>(wpt), w,
-                                                          w_dtype, eps, act, D, dim);
-  else
-    SA_REQUIRE(false, "token_side_few: unknown dtype %d", dtype);
-  return check_launch("token_side_few");
 }
 
 extern "C" int sa_bias_add(void* x, int dtype, int64_t stride, const void* b, int b_dtype, int T, int N,

@@ -71,8 +71,6 @@ _SIGNATURES = {
     "sa_delta_rule": [_P, _I, _I, _I, _I, _P, _I, _P, _L, _P, _I, _P, _P],
     "sa_embed_sum": [_P, _P, _P, _I, _I, _P, _I, _I, _P, _I, _L, _L, _L, _P, _L, _P, _I, _I, _P, _I, _P],
     "sa_token_gate": [_P, _I, _L, _P, _P, _I, _L, _I, _I, _I, _I, _P],
-    "sa_token_side_few": [_P, _P, _P, _I, _L, _I, _P, _P, _P, _I, _F, _I, _I, _I, _I, _P],
-    "sa_token_side_few_takes": [_I, _I, _I],
     "sa_bias_add": [_P, _I, _L, _P, _I, _I, _I, _P],
     "sa_weighted_sum": [_P, _L, _F, _P, _L, _F, _I, _P, _L, _I, _I, _P],
     "sa_exp_gates": [_P, _L, _P, _I, _F, _I, _P, _L, _P, _I, _P, _P],

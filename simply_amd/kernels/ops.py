@@ -1097,34 +1097,6 @@ def token_gate_(z: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, col0
     return z
 
 
-def token_side_few_takes(num_tokens: int, width: int, dim: int) -> bool:
-    """Whether `token_side_few` takes a step of this many tokens."""
-    return bool(_lib.load().sa_token_side_few_takes(int(num_tokens), int(width), int(dim)))
-
-
-def token_side_few(h: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor, col0: int, gate_w: torch.Tensor,
-                   proj_wt: torch.Tensor, norm_w: torch.Tensor, eps: float, activation: int) -> torch.Tensor:
-    """The per-layer token input of a step of few tokens in one launch: x = h in the tables' type, g = act(gate_w x) *
-    table[tokens, col0 : col0 + dim], y = proj_wt^T g, h += y / sqrt(mean(y^2) + eps) * norm_w, in place.  gate_w and
-    proj_wt (the projection transposed) are row-major [dim, D] of the table's type; h float32 [T, D]."""
-    _dev(h, tokens, table, gate_w, proj_wt, norm_w)
-    T, D = h.shape
-    dim = gate_w.shape[0]
-    if h.dtype != torch.float32 or not h.is_contiguous():
-        raise KernelError("token_side_few: the residual stream must be contiguous float32")
-    _i32(tokens, "token_side_few: tokens", T)
-    if tuple(gate_w.shape) != (dim, D) or tuple(proj_wt.shape) != (dim, D) or not gate_w.is_contiguous() \
-            or not proj_wt.is_contiguous() or gate_w.dtype != table.dtype or proj_wt.dtype != table.dtype:
-        raise KernelError("token_side_few: both factors are row-major [dim, D] of the table's type")
-    if table.dim() != 2 or table.stride(1) != 1 or col0 < 0 or col0 + dim > table.shape[1]:
-        raise KernelError(f"token_side_few: columns {col0}..{col0 + dim} of a table {tuple(table.shape)}")
-    if norm_w.numel() != D or not norm_w.is_contiguous():
-        raise KernelError("token_side_few: the norm's weight does not match the width")
-    _lib.call("sa_token_side_few", _ptr(h), _ptr(tokens), _ptr(table), _code(table), table.stride(0), int(col0),
-              _ptr(gate_w), _ptr(proj_wt), _ptr(norm_w), _code(norm_w), float(eps), int(activation), T, D, dim, _stream())
-    return h
-
-
 def bias_add_(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     """x[t, :] += bias, in place (the sum in 32-bit)."""
     _dev(x, bias)

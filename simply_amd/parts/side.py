@@ -32,15 +32,9 @@ class TokenSide(StreamPart):
     def load(self, tensors):
         self.table = tensors["table"]
         self.gate, self.proj = as_product_weight(tensors["gate"]), as_product_weight(tensors["proj"])
-        # for steps of few tokens, one kernel does it all and reads both factors row by row
-        self.gate_rows, self.proj_rows = tensors["gate"].contiguous(), tensors["proj"].t().contiguous()
         self.norm = tensors["norm"].contiguous()
 
     def forward(self, h, ctx):
-        if ops.token_side_few_takes(h.shape[0], self.hidden_size, self.dim):
-            ops.token_side_few(h, ctx.tokens, self.table, self.column, self.gate_rows, self.proj_rows, self.norm, self.eps,
-                               self.activation_code)
-            return
         x = h if ctx.dtype == torch.float32 else ops.residual_add_norm(None, h, out_dtype=ctx.dtype)
         z = ops.gemm(x, self.gate)
         ops.token_gate_(z, ctx.tokens, self.table, self.column, self.activation_code)

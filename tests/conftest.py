@@ -33,7 +33,7 @@ def cpu_ops(monkeypatch):
     for name in ("embed", "rmsnorm", "add_rmsnorm", "rope_cache_write", "rope", "gather_rows", "fill_", "gemm",
                  "paged_attention", "sample", "score", "decode_attention_takes", "paged_attention_sink",
                  "residual_add_norm", "gated_heads", "activation_", "qk_norm_rope_cache_write", "short_conv_silu",
-                 "delta_prepare", "delta_inputs", "delta_rule", "embed_sum", "token_gate_", "token_side_few", "token_side_few_takes", "bias_add_", "weighted_sum",
+                 "delta_prepare", "delta_inputs", "delta_rule", "embed_sum", "token_gate_", "bias_add_", "weighted_sum",
                  "exp_gates", "linear_state", "normalized_readout", "route", "routed_experts"):
         monkeypatch.setattr(ops, name, getattr(torch_ops, name))
     return torch_ops

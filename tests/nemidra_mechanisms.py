@@ -260,9 +260,8 @@ def token_side_part(device, dtype):
 
     class Ctx:
         pass
-    for n in (21, 5, 1):   # many tokens: separate kernels; few: one launch
-        ctx = Ctx()
-        ctx.dtype, ctx.tokens = dtype, torch.tensor(tokens[:n], dtype=torch.int32, device=device)
-        h = x[:n].to(device).clone()
-        part.forward(h, ctx)
-        _close(h, want[:n], dtype, ("token side", n))
+    ctx = Ctx()
+    ctx.dtype, ctx.tokens = dtype, torch.tensor(tokens, dtype=torch.int32, device=device)
+    h = x.to(device).clone()
+    part.forward(h, ctx)
+    _close(h, want, dtype, "token side")

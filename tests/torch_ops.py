@@ -604,18 +604,3 @@ def routed_experts(x, experts, weights, gate_w, up_w, down_w, activation, *, sha
         s = _f(shared)
         out = out + (s * torch.sigmoid(_f(shared_gate)[:, :1]) if shared_gate is not None else s)
     return out.to(out_dtype or x.dtype)
-
-
-def token_side_few_takes(num_tokens, width, dim):
-    return num_tokens <= 16 and dim <= 256 and width <= 12288
-
-
-def token_side_few(h, tokens, table, col0, gate_w, proj_wt, norm_w, eps, activation):
-    T = table.dtype
-    x = _f(h.to(T))
-    z = _f((x @ _f(gate_w).T).to(T))
-    g = _f((_activation(activation, z) * _f(table[tokens.long()][:, col0:col0 + gate_w.shape[0]])).to(T))
-    y = _f((g @ _f(proj_wt)).to(T))
-    y = y * torch.rsqrt((y * y).mean(-1, keepdim=True) + eps) * _f(norm_w)
-    h.copy_((_f(h) + y).to(torch.float32))
-    return h
