@@ -15,6 +15,8 @@
 // position of the first); what earlier steps left is the slot's state.  Gates, decays, sums and the state are 32-bit;
 // q, k and v are read from the projection in its own element type.  Sums run in an order that depends on the sizes
 // alone, so a token's result does not depend on how the tokens are cut into steps or on the batch.
+#include <type_traits>
+
 #include "api.h"
 #include "common.h"
 
@@ -115,7 +117,9 @@ __global__ __launch_bounds__(256) void linear_state_kernel(
         float a = ok ? gates[t * gates_stride + h * dk + d] : 0.f;
         if (ok && inv_tau > 0.f) {
           if (gate_bias != nullptr) a += load_f(gate_bias, bias_dtype, h * dk + d);
-          a = expf(log_sigmoid(a) * inv_tau);
+          // (a bfloat16 run takes the hardware's exponential and logarithm, a 32-bit run the library's)
+          if constexpr (sizeof(XT) == 2) a = __expf((fminf(a, 0.f) - __logf(1.f + __expf(-fabsf(a)))) * inv_tau);
+          else a = expf(log_sigmoid(a) * inv_tau);
         }
         pa[i] = a;
       }
@@ -148,13 +152,15 @@ __global__ __launch_bounds__(256) void linear_state_kernel(
     __syncthreads();
     if (t0 + kStateTokens < count) fetch(t0 + kStateTokens);
     // four tokens at a time: their updates follow one another, their sums across the lanes run side by side (a wave
-    // issues in order, and one such sum alone is a chain of dependent steps that nothing else covers)
-    for (int j0 = 0; j0 < tn; j0 += 4) {
+    // issues in order, and one such sum alone is a chain of dependent steps that nothing else covers).  A whole tile
+    // runs without a test per token, so that the reads of its operands can be asked for ahead of their use.
+    auto group = [&](int j0, auto whole) __attribute__((always_inline)) {
+      constexpr bool WHOLE = decltype(whole)::value;
       float o[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int j = j0 + i;
-        if (j < tn) {   // (uniform)
+        if (WHOLE || j < tn) {   // (uniform)
           float u = vs[j][tid / LPC], a0 = 1.f;
           if constexpr (SCALAR) {
             a0 = cs[j][0];
@@ -175,9 +181,15 @@ __global__ __launch_bounds__(256) void linear_state_kernel(
       if (live && part == 0) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (j0 + i < tn)
+          if (WHOLE || j0 + i < tn)
             out[static_cast<size_t>(first + t0 + j0 + i) * (static_cast<size_t>(H) * CT) + static_cast<size_t>(h) * CT + col] = o[i];
       }
+    };
+    if (tn == kStateTokens) {
+#pragma unroll
+      for (int j0 = 0; j0 < kStateTokens; j0 += 4) group(j0, std::true_type{});
+    } else {
+      for (int j0 = 0; j0 < tn; j0 += 4) group(j0, std::false_type{});
     }
   }
 #pragma unroll
