@@ -298,8 +298,9 @@ class FeedForward(Part):
 class StreamPart(Part):
     """A part at a block's end that reads and updates the residual stream itself."""
 
-    def forward(self, h: torch.Tensor, ctx: Any) -> None:
-        """h: float32 [T, D] residual stream, updated in place."""
+    def forward(self, h: torch.Tensor, ctx: Any, x: "torch.Tensor | None" = None) -> None:
+        """h: float32 [T, D] residual stream, updated in place.  x: the same stream in the activation type, if the
+        caller has it already."""
         raise NotImplementedError
 
 

@@ -12,6 +12,10 @@ import torch
 from ..kernels import ops
 from ..registry import BLOCKS
 from .base import Block, PendingNorm
+from .norm import NoNorm
+
+#: stands for "no norm follows": the kernel of the last residual sum then hands the stream on in the activation type
+_HAND_ON = NoNorm()
 
 
 @BLOCKS.register("sandwich")
@@ -44,8 +48,9 @@ class SandwichBlock(Block):
             both = part.defers_sum and getattr(norm, "adds_partial_sums", False) and ctx.dtype == torch.bfloat16
             return {"defer_sum": True} if both else {}
 
-        # (parts behind the feed-forward change the stream once more: the next block's norm comes after them)
-        after = None if self.extras else next_norm
+        # (parts behind the feed-forward change the stream once more: the next block's norm comes after them; they read
+        # the stream in the activation type, which the kernel of the last sum hands on)
+        after = _HAND_ON if self.extras else next_norm
         y = self.mixer.forward(normed, ctx, cache, **defer(self.mixer, n["post_mixer"]))
         if self.feed_forward is None:
             normed_next = n["post_mixer"].add_into(h, y, after, ctx.dtype)
@@ -54,8 +59,8 @@ class SandwichBlock(Block):
             y = self.feed_forward.forward(normed, ctx, **defer(self.feed_forward, n["post_ffn"]))
             normed_next = n["post_ffn"].add_into(h, y, after, ctx.dtype)
         if self.extras:
-            for part in self.extras:
-                part.forward(h, ctx)
+            for k, part in enumerate(self.extras):
+                part.forward(h, ctx, x=normed_next if k == 0 else None)
             normed_next = next_norm.forward(h, ctx.dtype) if next_norm is not None else None
         return h, normed_next
 
@@ -73,18 +78,17 @@ class SandwichBlock(Block):
         y = self.mixer.forward(give(self.mixer, x), ctx, cache)
         if isinstance(x, PendingNorm):
             h = x.settle()
-        if self.feed_forward is None:
-            x = PendingNorm(h, y, n["post_mixer"], next_norm, ctx.dtype)
-        else:
+        last = "post_mixer"
+        if self.feed_forward is not None:
             x = PendingNorm(h, y, n["post_mixer"], n["pre_ffn"], ctx.dtype)
             y = self.feed_forward.forward(give(self.feed_forward, x), ctx)
             h = x.settle()
-            x = PendingNorm(h, y, n["post_ffn"], next_norm, ctx.dtype)
+            last = "post_ffn"
         if not self.extras:
-            return h, x
-        h = x.settle()
-        for part in self.extras:
-            part.forward(h, ctx)
+            return h, PendingNorm(h, y, n[last], next_norm, ctx.dtype)
+        handed = n[last].add_into(h, y, _HAND_ON, ctx.dtype)
+        for k, part in enumerate(self.extras):
+            part.forward(h, ctx, x=handed if k == 0 else None)
         return h, PendingNorm(h, None, None, next_norm, ctx.dtype)
 
 

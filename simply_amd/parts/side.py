@@ -34,8 +34,9 @@ class TokenSide(StreamPart):
         self.gate, self.proj = as_product_weight(tensors["gate"]), as_product_weight(tensors["proj"])
         self.norm = tensors["norm"].contiguous()
 
-    def forward(self, h, ctx):
-        x = h if ctx.dtype == torch.float32 else ops.residual_add_norm(None, h, out_dtype=ctx.dtype)
+    def forward(self, h, ctx, x=None):
+        if x is None:
+            x = h if ctx.dtype == torch.float32 else ops.residual_add_norm(None, h, out_dtype=ctx.dtype)
         z = ops.gemm(x, self.gate)
         ops.token_gate_(z, ctx.tokens, self.table, self.column, self.activation_code)
         y = ops.gemm(z, self.proj)
