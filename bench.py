@@ -463,12 +463,12 @@ def nemidra_config(size: dict, layers: int, positions: int) -> dict:
                    "shared": {"ff": ff // 4}}
         if i % 4 == 3:
             mixer = {"left": {"heads": H, "kv_heads": K, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": 1024}},
-                     "right": {"heads": H // 2, "dim": d, "vdim": d, "gate_cap": 15.0}, "left_scale": 1.0, "right_scale": 1.0}
+                     "right": {"heads": H // 2, "dim": d, "vdim": d, "gate_cap": 10.0}, "left_scale": 1.0, "right_scale": 1.0}
             out.append({"type": "parallel", "mixer": mixer, "mlp": mlp})
         else:
-            out.append({"type": "gla", "mixer": {"heads": H, "dim": d, "vdim": d, "tau": 16.0, "rank": 64}, "mlp": mlp})
+            out.append({"type": "gla", "mixer": {"heads": H, "dim": d, "vdim": d, "tau": 8.0, "rank": 64}, "mlp": mlp})
     return {"architecture": "Nemidra", "vocab": size["vocab"], "width": W, "norm": {"eps": 1e-5}, "layers": out,
-            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}}, "max_positions": positions,
+            "embedding": {"bigram": {"buckets": 65521, "mul_prev": 8191, "mul_cur": 127}}, "max_positions": positions,
             "token_side": {"dim": 64}, "logit_softcap": 30.0}
 
 

@@ -64,7 +64,7 @@ MIXED = config(83, 40, 1e-5, [
 #: what the others make unequal is equal or 1 here: one head, as many key heads as heads, every expert used, a loop
 #: that runs once and one that starts at layer 0, a window of 1, no pair table, no side input, no cap on the logits
 UNITS = config(31, 24, 1e-6, [
-    parallel((1, 1, 8, 8, 0.5, 1), (1, 4, 4, 15.0), 1.0, 1.0, mlp=moe(3, 3, 8, 2.0)),
+    parallel((1, 1, 8, 8, 0.5, 1), (1, 4, 4, 9.0), 1.0, 1.0, mlp=moe(3, 3, 8, 1.25)),
     gla(1, 4, 4, 1.0, 1),
     parallel((2, 2, 8, 4, 0.4, None), (1, 16, 8, 2.0), 1.0, 0.5, mlp=dense(16)),
 ], loop=(0, 2, 1), bigram=None, side=None, cap=None)
@@ -73,10 +73,10 @@ LOOP_FROM_START = config(40, 32, 1e-5, [gla(2, 8, 8, 4.0, 2, mlp=dense(24)),
                          positions=None)
 #: sizes in multiples of 32 and 64 (what fast kernels may take), still small
 ALIGNED = config(256, 128, 1e-5, [
-    gla(2, 64, 64, 16.0, 16, mlp=moe(8, 2, 64, 2.0, shared=64)),
-    parallel((4, 2, 64, 64, 0.125, 40), (2, 32, 64, 15.0), 1.2, 0.9, mlp=dense(256)),
-    gla(1, 128, 128, 16.0, 8),
-    parallel((8, 1, 128, 128, 0.09, 24), (1, 128, 32, 15.0), 1.0, 1.0, mlp=moe(4, 2, 128, 1.0)),
+    gla(2, 64, 64, 12.0, 16, mlp=moe(8, 2, 64, 1.75, shared=64)),
+    parallel((4, 2, 64, 64, 0.125, 48), (2, 32, 64, 12.0), 1.25, 0.85, mlp=dense(256)),
+    gla(1, 128, 128, 12.0, 8),
+    parallel((8, 1, 128, 128, 0.09, 24), (1, 128, 32, 9.0), 1.0, 1.0, mlp=moe(4, 2, 128, 1.0)),
 ], loop=(1, 3, 2), side=16)
 #: name -> (configuration, seed, standard deviation of the matrices, of the norms' weights and biases).  The wider model
 #: has smaller weights: with large ones its scores are so sharp that a bfloat16 run and the plain one part ways.
@@ -98,20 +98,20 @@ def drawn_config(seed: int) -> dict:
         if kind == "dense":
             return dense(r.choice([16, 40, 100]))
         experts = r.choice([2, 3, 6, 9])
-        return moe(experts, r.randint(1, min(experts, 3)), r.choice([8, 20, 36]), r.choice([0.5, 1.0, 2.0]),
+        return moe(experts, r.randint(1, min(experts, 3)), r.choice([8, 20, 36]), r.choice([0.5, 1.0, 1.5]),
                    shared=r.choice([None, 12, 24]))
 
     layers = []
     for _ in range(r.randint(2, 5)):
         if r.random() < 0.5:
             layers.append(gla(r.choice([1, 2, 3]), r.choice([4, 12, 16, 40, 72]), r.choice([4, 8, 20, 70]),
-                              r.choice([1.0, 4.0, 16.0]), r.choice([1, 2, 6]), mlp=mlp()))
+                              r.choice([1.0, 4.0, 12.0]), r.choice([1, 2, 6]), mlp=mlp()))
         else:
             kv = r.choice([1, 2, 3])
             left = (kv * r.choice([1, 2, 4]), kv, r.choice([8, 12, 32, 48]), r.choice([4, 8, 24]),
                     r.choice([0.2, 0.5]), r.choice([None, 1, 3, 4, 9, 16, 30]))
-            right = (r.choice([1, 2, 3]), r.choice([4, 8, 24, 40]), r.choice([4, 12, 33]), r.choice([3.0, 15.0]))
-            layers.append(parallel(left, right, r.choice([0.5, 1.0, 1.2]), r.choice([0.9, 1.0]), mlp=mlp()))
+            right = (r.choice([1, 2, 3]), r.choice([4, 8, 24, 40]), r.choice([4, 12, 33]), r.choice([3.0, 12.0]))
+            layers.append(parallel(left, right, r.choice([0.5, 1.0, 1.3]), r.choice([0.8, 1.0]), mlp=mlp()))
     n = len(layers)
     loop = None
     if r.random() < 0.7:

@@ -90,12 +90,12 @@ def test_plain_recurrences_in_portions():
     w |= {"p.i.b": torch.zeros(H, dtype=torch.float64), "p.f.b": torch.ones(H, dtype=torch.float64),
           "p.norm": torch.ones(H * dv, dtype=torch.float64)}
     h = torch.randn(T, D, generator=g, dtype=torch.float64)
-    m = {"heads": H, "dim": dk, "vdim": dv, "gate_cap": 15.0}
+    m = {"heads": H, "dim": dk, "vdim": dv, "gate_cap": 11.0}
     got = plain.mlstm(w, "p.", m, h, 1e-6)
     q = (h @ w["p.q"].T).view(T, H, dk) * dk ** -0.5
     k, v = (h @ w["p.k"].T).view(T, H, dk), (h @ w["p.v"].T).view(T, H, dv)
-    ig = 15.0 * torch.tanh((h @ w["p.i"].T) / 15.0)
-    fg = torch.nn.functional.logsigmoid(15.0 * torch.tanh((h @ w["p.f"].T + 1.0) / 15.0))
+    ig = 11.0 * torch.tanh((h @ w["p.i"].T) / 11.0)
+    fg = torch.nn.functional.logsigmoid(11.0 * torch.tanh((h @ w["p.f"].T + 1.0) / 11.0))
     out = torch.zeros(T, H, dv, dtype=torch.float64)
     for a in range(H):
         S, n, logm = torch.zeros(dk, dv, dtype=torch.float64), torch.zeros(dk, dtype=torch.float64), 0.0
