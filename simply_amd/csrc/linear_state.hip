@@ -101,7 +101,8 @@ __global__ __launch_bounds__(256) void linear_state_kernel(
     s[r] = (live && i < dk) ? S[static_cast<size_t>(col) * dk + i] : 0.f;
   }
   constexpr int PQ = kStateTokens * DK / 256, PV = (kStateTokens * COLS + 255) / 256;
-  float pq[PQ], pk[PQ], pa[SCALAR ? 1 : PQ], pv[PV], pc = 0.f;
+  float pq[PQ], pk[PQ], pa[SCALAR ? 1 : PQ], pb[SCALAR ? 1 : PQ], pv[PV], pc = 0.f;
+  bool pok[SCALAR ? 1 : PQ];
   auto fetch = [&](int t0) __attribute__((always_inline)) {
     const int tn = count - t0 < kStateTokens ? count - t0 : kStateTokens;
 #pragma unroll
@@ -113,15 +114,11 @@ __global__ __launch_bounds__(256) void linear_state_kernel(
       pq[i] = ok ? to_float(row[q_at + h * dk + d]) * q_mult : 0.f;
       pk[i] = ok ? to_float(row[k_at + h * dk + d]) : 0.f;
       if constexpr (!SCALAR) {
-        // inv_tau > 0: the gates are z, and the decay is sigmoid(z + bias)^(1 / tau)
-        float a = ok ? gates[t * gates_stride + h * dk + d] : 0.f;
-        if (ok && inv_tau > 0.f) {
-          if (gate_bias != nullptr) a += load_f(gate_bias, bias_dtype, h * dk + d);
-          // (a bfloat16 run takes the hardware's exponential and logarithm, a 32-bit run the library's)
-          if constexpr (sizeof(XT) == 2) a = __expf((fminf(a, 0.f) - __logf(1.f + __expf(-fabsf(a)))) * inv_tau);
-          else a = expf(log_sigmoid(a) * inv_tau);
-        }
-        pa[i] = a;
+        // (with inv_tau > 0 the gates are z and the bias rides along: the decay is computed when the tile is put into
+        // LDS, a tile later, so that nothing waits for these loads here)
+        pa[i] = ok ? gates[t * gates_stride + h * dk + d] : 0.f;
+        if (inv_tau > 0.f) pb[i] = (ok && gate_bias != nullptr) ? load_f(gate_bias, bias_dtype, h * dk + d) : 0.f;
+        pok[i] = ok;
       }
     }
 #pragma unroll
@@ -141,7 +138,17 @@ __global__ __launch_bounds__(256) void linear_state_kernel(
       const int idx = tid + i * 256;
       qs[idx / DK][idx % DK] = pq[i];
       ks[idx / DK][idx % DK] = pk[i];
-      if constexpr (!SCALAR) as[idx / DK][idx % AD] = pa[i];
+      if constexpr (!SCALAR) {
+        // a = sigmoid(z + bias)^(1 / tau): a bfloat16 run takes the hardware's exponential and logarithm, a 32-bit
+        // run the library's
+        float a = pa[i];
+        if (inv_tau > 0.f && pok[i]) {
+          a += pb[i];
+          if constexpr (sizeof(XT) == 2) a = __expf((fminf(a, 0.f) - __logf(1.f + __expf(-fabsf(a)))) * inv_tau);
+          else a = expf(log_sigmoid(a) * inv_tau);
+        }
+        as[idx / DK][idx % AD] = a;
+      }
     }
 #pragma unroll
     for (int i = 0; i < PV; ++i) {
