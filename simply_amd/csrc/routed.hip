@@ -146,7 +146,28 @@ __global__ __launch_bounds__(256) void expert_product_kernel(
     floatx4 accg[RT], accu[RT];
 #pragma unroll
     for (int s = 0; s < RT; ++s) accg[s] = accu[s] = floatx4{0.f, 0.f, 0.f, 0.f};
-    for (int kt = 0; kt < Kt; ++kt) {
+    // Whole k tiles of aligned rows, four at a time: their loads are all asked for before the first product (few
+    // waves run on a SIMD here, so a wave covers its own waits), the products in the order of k.
+    int kt = 0;
+    if (aligned && RT == 1) {
+      const bf16* src = reinterpret_cast<const bf16*>(arow[0]) + kq * 8;
+      constexpr int kAhead = 4;
+      for (; kt + kAhead <= K / 32; kt += kAhead) {
+        bf16x8 gv[kAhead], uv[kAhead], av[kAhead];
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+          gv[i] = load8(g + static_cast<size_t>(kt + i) * 512);
+          if constexpr (GATED) uv[i] = load8(u + static_cast<size_t>(kt + i) * 512);
+          av[i] = load8(src + (kt + i) * 32);
+        }
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) {
+          accg[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gv[i], av[i], accg[0], 0, 0, 0);
+          if constexpr (GATED) accu[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uv[i], av[i], accu[0], 0, 0, 0);
+        }
+      }
+    }
+    for (; kt < Kt; ++kt) {
       const int k = kt * 32 + kq * 8;
       const bf16x8 gv = load8(g + static_cast<size_t>(kt) * 512);
       bf16x8 uv = gv;
